@@ -47,21 +47,33 @@ void launch_hy_window_prep(void*, int, int, int, int, int, const void*, const fl
 int hy_window_rows_cap(int, int, int, bool);
 void launch_hy_window_attention(const void*, int, const void*, const void*, const int32_t*, int, const int32_t*,
                                 const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
-                                int, int, bool, int, float*, float*, int64_t, hipStream_t);
-int hy_window_nsplit(bool, int, int, int, int, int, int, int, int, int, int);
-void launch_hy_short_conv(const void*, int, const float*, const int32_t*, const int32_t*, const int32_t*, const int32_t*,
-                          void*, void*, int, int, int, int, bool, bool, hipStream_t);
+                                int, int, int, bool, int, float*, float*, int64_t, hipStream_t);
+int hy_window_nsplit(bool, int, int, int, int, int, int, int, int, int, int, int);
+void launch_hy_short_conv(const void*, int, const float*, const float*, const int32_t*, const int32_t*, const int32_t*,
+                          const int32_t*, void*, void*, int, int, int, int, bool, bool, hipStream_t);
 void launch_hy_delta_prep(const void*, int, const float*, const float*, float*, float*, float*, float*, int, int, int, int,
                           float, bool, hipStream_t);
 bool launch_hy_linear_scan(const void*, int, int, int, int, const float*, const float*, float, const float*, bool,
                            const float*, const int32_t*, const int32_t*, const int32_t*, float*, float*, int, int, int, int,
-                           int, int, bool, hipStream_t);
+                           int, int, const float*, bool, hipStream_t);
 void launch_hy_moe_route_topk(const void*, const void*, const float*, float*, int32_t*, float*, int, int, int, int, bool,
                               hipStream_t);
 void launch_hy_moe_glu_grouped(const uint16_t*, const int32_t*, const float*, const uint16_t*, const uint16_t*, uint16_t*,
                                int32_t*, uint16_t*, uint16_t*, int, int, int, int, int, float, float, float, hipStream_t);
 void launch_hy_moe_glu_token(const void*, const int32_t*, const float*, const void*, const void*, void*, int, int, int,
                              int, int, float, float, float, bool, bool, hipStream_t);
+void launch_hy_add_rms_norm(const void*, const void*, const float*, const float*, float*, const float*, void*, int, int,
+                            float, int, bool, hipStream_t);
+void launch_hy_token_gate(const void*, const int32_t*, const void*, int, int, void*, int, int, bool, hipStream_t);
+void launch_hy_ssm_prep(const float*, const float*, float*, float*, int, int, hipStream_t);
+void launch_hy_gated_group_norm(const float*, const void*, int, int, const float*, const void*, int, int, const float*,
+                                void*, int, int, int, int, float, bool, hipStream_t);
+int hy_rglru_chunks(int);
+void launch_hy_rglru_scan(const void*, const float*, const float*, float, const void*, int, int, const int32_t*,
+                          const int32_t*, const int32_t*, float*, float*, float*, void*, int, int, int, int, int, bool,
+                          hipStream_t);
+void launch_hy_moe_route_group(const void*, const void*, float*, int32_t*, float*, int, int, int, int, int, int, float, bool,
+                               hipStream_t);
 }  // namespace chronos
 
 namespace {
@@ -339,8 +351,8 @@ Tensor hy_head_norm_gate(const Tensor& o, const Tensor& src, int64_t g_off, cons
 
 Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, const c10::optional<Tensor>& v_first,
                       const c10::optional<Tensor>& lam, const Tensor& pos, const Tensor& tok_seq, const Tensor& block_table,
-                      const Tensor& q_norm, const Tensor& k_norm, double eps, const c10::optional<Tensor>& cos_sin,
-                      int64_t dims, Tensor& kc, Tensor& vc, bool emit_v) {
+                      const c10::optional<Tensor>& q_norm, const c10::optional<Tensor>& k_norm, double eps,
+                      const c10::optional<Tensor>& cos_sin, int64_t dims, Tensor& kc, Tensor& vc, bool emit_v) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
     same_act(qkv, kc, "window_prep: the caches hold the activation dtype");
     same_act(qkv, vc, "window_prep: the caches hold the activation dtype");
@@ -350,8 +362,11 @@ Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, 
     need(kc.size(2) == G && kc.size(3) == D && vc.size(2) == G && vc.size(3) == Dv && vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "window_prep: cache shapes");
     i32(pos, "window_prep: pos"); i32(tok_seq, "window_prep: tok_seq"); i32(block_table, "window_prep: block_table");
     need(pos.numel() == T && tok_seq.numel() == T && block_table.dim() == 2, "window_prep: per-token metadata");
-    flt(q_norm, "window_prep: float32 norm weight"); flt(k_norm, "window_prep: float32 norm weight");
-    need(q_norm.numel() == D && k_norm.numel() == D, "window_prep: norm weights [D]");
+    need(q_norm.has_value() == k_norm.has_value(), "window_prep: queries and keys are normed together or not at all");
+    if (q_norm) {
+        flt(*q_norm, "window_prep: float32 norm weight"); flt(*k_norm, "window_prep: float32 norm weight");
+        need(q_norm->numel() == D && k_norm->numel() == D, "window_prep: norm weights [D]");
+    }
     need(dims >= 0 && dims % 2 == 0 && dims <= D, "window_prep: rotated columns");
     if (dims > 0) {
         need(cos_sin.has_value(), "window_prep: rotation needs the cos/sin table");
@@ -369,7 +384,8 @@ Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, 
     chronos::launch_hy_window_prep(qkv.data_ptr(), (int)qkv.size(1), (int)H, (int)G, (int)D, (int)Dv,
                                    v_first ? v_first->data_ptr() : nullptr, v_first ? lam->data_ptr<float>() : nullptr,
                                    pos.data_ptr<int32_t>(), tok_seq.data_ptr<int32_t>(), block_table.data_ptr<int32_t>(),
-                                   (int)block_table.size(1), q_norm.data_ptr<float>(), k_norm.data_ptr<float>(), (float)eps,
+                                   (int)block_table.size(1), q_norm ? q_norm->data_ptr<float>() : nullptr,
+                                   k_norm ? k_norm->data_ptr<float>() : nullptr, (float)eps,
                                    dims > 0 ? cos_sin->data_ptr<float>() : nullptr, (int)dims, kc.data_ptr(), vc.data_ptr(),
                                    (int)kc.size(1), emit_v ? v_out.data_ptr() : nullptr, (int)T, f32(qkv), stream());
     return v_out;
@@ -377,8 +393,8 @@ Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, 
 
 Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc, const Tensor& block_table,
                            const Tensor& q_start, const Tensor& pos, const c10::optional<Tensor>& sink,
-                           const c10::optional<Tensor>& gate, double scale, int64_t window, int64_t keep, int64_t H,
-                           int64_t max_q) {
+                           const c10::optional<Tensor>& gate, double scale, int64_t window, int64_t keep, int64_t chunk,
+                           int64_t H, int64_t max_q) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
     same_act(qkv, kc, "window_attention: queries and caches in one activation dtype");
     same_act(qkv, vc, "window_attention: queries and caches in one activation dtype");
@@ -389,14 +405,14 @@ Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc
     need(chronos::hy_window_rows_cap((int)(H / G), (int)D, (int)Dv, f32(qkv)) > 0, "window_attention: a key tile and a group's query rows must fit the LDS");
     i32(block_table, "window_attention: block_table"); i32(q_start, "window_attention: q_start"); i32(pos, "window_attention: pos");
     const int64_t B = q_start.numel() - 1;
-    need(block_table.dim() == 2 && block_table.size(0) >= B && pos.numel() == T && window >= 0 && keep >= 0, "window_attention: metadata");
+    need(block_table.dim() == 2 && block_table.size(0) >= B && pos.numel() == T && window >= 0 && keep >= 0 && chunk >= 0, "window_attention: metadata");
     if (sink) { flt(*sink, "window_attention: float32 sinks"); need(sink->numel() == H, "window_attention: sink [H]"); }
     if (gate) { flt(*gate, "window_attention: float32 gate"); need(gate->numel() == T * H, "window_attention: gate [T, H]"); }
     auto out = at::empty({T, H * Dv}, qkv.options());
     if (T == 0 || B <= 0) return out;
     const int mq = (int)std::max<int64_t>(1, max_q);
     const int nsplit = chronos::hy_window_nsplit(f32(qkv), (int)qkv.size(1), (int)B, mq, (int)H, (int)G, (int)D, (int)Dv,
-                                                 (int)window, (int)keep, (int)(block_table.size(1) * kc.size(1)));
+                                                 (int)window, (int)keep, (int)chunk, (int)(block_table.size(1) * kc.size(1)));
     Tensor part_o, part_ml;
     if (nsplit > 1) {
         part_o = at::empty({T * H * nsplit, Dv}, qkv.options().dtype(at::kFloat));
@@ -407,24 +423,27 @@ Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc
                                         q_start.data_ptr<int32_t>(), pos.data_ptr<int32_t>(),
                                         sink ? sink->data_ptr<float>() : nullptr, gate ? gate->data_ptr<float>() : nullptr,
                                         out.data_ptr(), (int)B, mq, (int)H, (int)G, (int)D, (int)Dv, (int)kc.size(1),
-                                        (float)scale, (int)window, (int)keep, f32(qkv), nsplit,
+                                        (float)scale, (int)window, (int)keep, (int)chunk, f32(qkv), nsplit,
                                         nsplit > 1 ? part_o.data_ptr<float>() : nullptr,
                                         nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, T * H, stream());
     return out;
 }
 
 Tensor hy_short_conv(const Tensor& x, const Tensor& w, const Tensor& tok_seq, const Tensor& q_start, const Tensor& pos0,
-                     const Tensor& slots, Tensor& hist, bool silu) {
+                     const Tensor& slots, Tensor& hist, bool silu, const c10::optional<Tensor>& bias, int64_t x_off) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
     same_act(x, hist, "short_conv: the history holds the activation dtype");
     flt(w, "short_conv: float32 taps");
     need(x.dim() == 2 && x.is_contiguous() && w.dim() == 2 && hist.dim() == 3 && hist.is_contiguous(), "short_conv: layouts");
     const int64_t T = x.size(0), C = w.size(0), K = w.size(1), B = slots.numel();
-    need(C <= x.size(1) && K >= 1 && hist.size(1) == K - 1 && hist.size(2) == C, "short_conv: channels / taps / history");
+    need(x_off >= 0 && x_off + C <= x.size(1) && K >= 1 && hist.size(1) == K - 1 && hist.size(2) == C, "short_conv: channels / taps / history");
+    if (bias) { flt(*bias, "short_conv: float32 bias"); need(bias->numel() == C, "short_conv: bias [C]"); }
     i32(tok_seq, "short_conv: tok_seq"); i32(q_start, "short_conv: q_start"); i32(pos0, "short_conv: pos0"); i32(slots, "short_conv: slots");
     need(tok_seq.numel() == T && q_start.numel() == B + 1 && pos0.numel() == B, "short_conv: metadata");
     auto y = at::empty({T, C}, x.options());
-    chronos::launch_hy_short_conv(x.data_ptr(), (int)x.size(1), w.data_ptr<float>(), tok_seq.data_ptr<int32_t>(),
+    const char* xp = (const char*)x.data_ptr() + x_off * x.element_size();
+    chronos::launch_hy_short_conv(xp, (int)x.size(1), w.data_ptr<float>(), bias ? bias->data_ptr<float>() : nullptr,
+                                  tok_seq.data_ptr<int32_t>(),
                                   q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(), slots.data_ptr<int32_t>(),
                                   hist.data_ptr(), y.data_ptr(), (int)T, (int)B, (int)C, (int)K, silu, f32(x), stream());
     return y;
@@ -448,7 +467,7 @@ std::tuple<Tensor, Tensor, Tensor, Tensor> hy_delta_prep(const Tensor& y, const 
 Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t v_off, const c10::optional<Tensor>& qscale,
                       const c10::optional<Tensor>& kscale, double q_mul, const Tensor& decay,
                       const c10::optional<Tensor>& beta, const Tensor& q_start, const Tensor& pos0, const Tensor& slots,
-                      Tensor& S, int64_t HK, int64_t H, int64_t D, int64_t Dv) {
+                      Tensor& S, int64_t HK, int64_t H, int64_t D, int64_t Dv, const c10::optional<Tensor>& vscale) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
     need(is_act(proj) && proj.dim() == 2 && proj.is_contiguous(), "linear_scan: proj [T, C]");
     const int64_t T = proj.size(0), C = proj.size(1), B = slots.numel();
@@ -460,6 +479,7 @@ Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t 
     if (qscale) { flt(*qscale, "linear_scan: qscale"); need(qscale->numel() == T * HK, "linear_scan: qscale [T, HK]"); }
     if (kscale) { flt(*kscale, "linear_scan: kscale"); need(kscale->numel() == T * HK, "linear_scan: kscale [T, HK]"); }
     if (beta) { flt(*beta, "linear_scan: beta"); need(beta->numel() == T * H, "linear_scan: beta [T, H]"); }
+    if (vscale) { flt(*vscale, "linear_scan: vscale"); need(vscale->numel() == T * H && !beta, "linear_scan: vscale [T, H], without the delta correction"); }
     i32(q_start, "linear_scan: q_start"); i32(pos0, "linear_scan: pos0"); i32(slots, "linear_scan: slots");
     need(q_start.numel() == B + 1 && pos0.numel() == B, "linear_scan: q_start [B+1], pos0 [B], slots [B]");
     flt(S, "linear_scan: S");
@@ -471,7 +491,7 @@ Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t 
         kscale ? kscale->data_ptr<float>() : nullptr, (float)q_mul, decay.data_ptr<float>(), chd,
         beta ? beta->data_ptr<float>() : nullptr, q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(),
         slots.data_ptr<int32_t>(), S.data_ptr<float>(), o.data_ptr<float>(), (int)T, (int)B, (int)HK, (int)H, (int)D, (int)Dv,
-        f32(proj), stream());
+        vscale ? vscale->data_ptr<float>() : nullptr, f32(proj), stream());
     TORCH_CHECK(ok, "chronos hybrid op: linear_scan keeps a state column in registers, D <= 256 (got ", D, ")");
     return o;
 }
@@ -526,6 +546,120 @@ Tensor hy_moe_glu_ffn(const Tensor& h, const Tensor& idx, const Tensor& wt, cons
     return out;
 }
 
+Tensor hy_add_rms_norm(const Tensor& y, Tensor& x, const c10::optional<Tensor>& w_out, double eps, bool out_f32,
+                       const c10::optional<Tensor>& y2, const c10::optional<Tensor>& gate2,
+                       const c10::optional<Tensor>& w_y, bool emit) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "add_rms_norm: float32 residual");
+    need(x.dim() == 2 && is_act(y) && y.is_contiguous() && y.sizes() == x.sizes() && f32(y) == out_f32, "add_rms_norm: y [T, d] in the activation dtype");
+    const int64_t T = x.size(0), d = x.size(1);
+    if (w_out) { flt(*w_out, "add_rms_norm: float32 weight"); need(w_out->numel() == d, "add_rms_norm: weight size"); }
+    if (w_y) { flt(*w_y, "add_rms_norm: float32 weight"); need(w_y->numel() == d, "add_rms_norm: weight size"); }
+    need(y2.has_value() == gate2.has_value(), "add_rms_norm: a second addend comes with its gate");
+    if (y2) {
+        same_act(y, *y2, "add_rms_norm: y2 in the activation dtype");
+        need(y2->is_contiguous() && y2->sizes() == x.sizes(), "add_rms_norm: y2 shape");
+        flt(*gate2, "add_rms_norm: float32 gate");
+        need(gate2->numel() == T, "add_rms_norm: one gate per row");
+    }
+    const int mode = !emit ? 0 : (w_out ? 2 : 1);
+    // float activations read the updated stream itself
+    const bool has_h = mode == 2 || (mode == 1 && !out_f32);
+    Tensor h = has_h ? at::empty({T, d}, x.options().dtype(out_f32 ? at::kFloat : at::kBFloat16)) : at::empty({0}, x.options());
+    chronos::launch_hy_add_rms_norm(y.data_ptr(), y2 ? y2->data_ptr() : nullptr, gate2 ? gate2->data_ptr<float>() : nullptr,
+                                    w_y ? w_y->data_ptr<float>() : nullptr, x.data_ptr<float>(),
+                                    w_out ? w_out->data_ptr<float>() : nullptr, has_h ? h.data_ptr() : nullptr, (int)T, (int)d,
+                                    (float)eps, has_h ? mode : 0, out_f32, stream());
+    return h;
+}
+
+Tensor hy_token_gate(const Tensor& a, const Tensor& ids, const Tensor& table, int64_t col0) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(a.device());
+    same_act(a, table, "token_gate: projection and table in one activation dtype");
+    need(a.dim() == 2 && a.is_contiguous() && table.dim() == 2 && table.is_contiguous(), "token_gate: layouts");
+    i32(ids, "token_gate: ids");
+    need(ids.numel() == a.size(0) && col0 >= 0 && col0 + a.size(1) <= table.size(1), "token_gate: ids [T], columns inside the table");
+    auto out = at::empty_like(a);
+    chronos::launch_hy_token_gate(a.data_ptr(), ids.data_ptr<int32_t>(), table.data_ptr(), (int)table.size(1), (int)col0,
+                                  out.data_ptr(), (int)a.size(0), (int)a.size(1), f32(a), stream());
+    return out;
+}
+
+std::tuple<Tensor, Tensor> hy_ssm_prep(const Tensor& dt_pre, const Tensor& a_log) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(dt_pre.device());
+    flt(dt_pre, "ssm_prep: float32 pre-activations"); flt(a_log, "ssm_prep: float32 A_log");
+    need(dt_pre.dim() == 2 && dt_pre.size(1) == a_log.numel(), "ssm_prep: dt_pre [T, H], a_log [H]");
+    auto decay = at::empty_like(dt_pre), dt = at::empty_like(dt_pre);
+    chronos::launch_hy_ssm_prep(dt_pre.data_ptr<float>(), a_log.data_ptr<float>(), decay.data_ptr<float>(),
+                                dt.data_ptr<float>(), (int)dt_pre.size(0), (int)dt_pre.size(1), stream());
+    return {decay, dt};
+}
+
+Tensor hy_gated_group_norm(const Tensor& o, const Tensor& skip_src, int64_t skip_off, const Tensor& skip_w,
+                           const Tensor& gate_src, int64_t g_off, const Tensor& w, int64_t groups, double eps, bool out_f32) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
+    flt(o, "gated_group_norm: float32 read-out"); flt(w, "gated_group_norm: float32 weight"); flt(skip_w, "gated_group_norm: float32 skip weights");
+    need(o.dim() == 3, "gated_group_norm: o [T, H, Dv]");
+    const int64_t T = o.size(0), H = o.size(1), Dv = o.size(2), n = H * Dv;
+    same_act(skip_src, gate_src, "gated_group_norm: sources in one activation dtype");
+    need(f32(gate_src) == out_f32 && skip_src.dim() == 2 && gate_src.dim() == 2 && skip_src.is_contiguous() && gate_src.is_contiguous() &&
+         skip_src.size(0) == T && gate_src.size(0) == T, "gated_group_norm: sources [T, C]");
+    need(skip_off >= 0 && skip_off + n <= skip_src.size(1) && g_off >= 0 && g_off + n <= gate_src.size(1), "gated_group_norm: column ranges");
+    need(w.numel() == n && skip_w.numel() == H && groups >= 1 && n % groups == 0, "gated_group_norm: weight [H Dv], skip [H], equal groups");
+    auto y = at::empty({T, n}, gate_src.options());
+    chronos::launch_hy_gated_group_norm(o.data_ptr<float>(), skip_src.data_ptr(), (int)skip_src.size(1), (int)skip_off,
+                                        skip_w.data_ptr<float>(), gate_src.data_ptr(), (int)gate_src.size(1), (int)g_off,
+                                        w.data_ptr<float>(), y.data_ptr(), (int)T, (int)n, (int)groups, (int)Dv, (float)eps,
+                                        out_f32, stream());
+    return y;
+}
+
+Tensor hy_rglru_scan(const Tensor& u, const Tensor& gates, const Tensor& sp, double c, const Tensor& ysrc, int64_t y_off,
+                     const Tensor& q_start, const Tensor& pos0, const Tensor& slots, Tensor& S, int64_t max_q) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(u.device());
+    same_act(u, ysrc, "rglru_scan: branches in one activation dtype");
+    need(u.dim() == 2 && u.is_contiguous() && ysrc.dim() == 2 && ysrc.is_contiguous() && ysrc.size(0) == u.size(0), "rglru_scan: layouts");
+    const int64_t T = u.size(0), W = u.size(1), B = slots.numel();
+    flt(gates, "rglru_scan: float32 gate pre-activations"); flt(sp, "rglru_scan: float32 decay parameter"); flt(S, "rglru_scan: S");
+    need(gates.dim() == 3 && gates.size(1) == T && gates.size(0) >= 1 && W % gates.size(0) == 0 &&
+         gates.size(2) == 2 * (W / gates.size(0)), "rglru_scan: gates [blocks, T, 2 W / blocks]");
+    need(sp.numel() == W && y_off >= 0 && y_off + W <= ysrc.size(1) && S.dim() == 2 && S.size(1) == W, "rglru_scan: widths");
+    i32(q_start, "rglru_scan: q_start"); i32(pos0, "rglru_scan: pos0"); i32(slots, "rglru_scan: slots");
+    need(q_start.numel() == B + 1 && pos0.numel() == B, "rglru_scan: q_start [B+1], pos0 [B], slots [B]");
+    auto out = at::empty_like(u);
+    if (T == 0 || B == 0) return out;
+    const int nch = chronos::hy_rglru_chunks((int)std::max<int64_t>(1, max_q > 0 ? max_q : T));
+    Tensor pq, init;
+    if (nch > 1) {
+        pq = at::empty({B, nch, 2, W}, S.options());
+        init = at::empty({B, W}, S.options());
+    }
+    chronos::launch_hy_rglru_scan(u.data_ptr(), gates.data_ptr<float>(), sp.data_ptr<float>(), (float)c, ysrc.data_ptr(),
+                                  (int)ysrc.size(1), (int)y_off, q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(),
+                                  slots.data_ptr<int32_t>(), S.data_ptr<float>(), nch > 1 ? pq.data_ptr<float>() : nullptr,
+                                  nch > 1 ? init.data_ptr<float>() : nullptr, out.data_ptr(), (int)T, (int)B, (int)W,
+                                  (int)(W / gates.size(0)), nch, f32(u), stream());
+    return out;
+}
+
+std::tuple<Tensor, Tensor> hy_moe_route_group(const Tensor& h, const Tensor& w, int64_t top, int64_t n_groups, int64_t keep,
+                                              double scale) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(h.device());
+    same_act(h, w, "moe_route_group: h and router in one activation dtype");
+    need(h.dim() == 2 && w.dim() == 2 && h.is_contiguous() && w.is_contiguous() && h.size(1) == w.size(1), "moe_route_group: shapes");
+    const int64_t N = w.size(0);
+    need(N <= 256 && n_groups >= 1 && n_groups <= 64 && N % n_groups == 0 && keep >= 1 && keep <= n_groups,
+         "moe_route_group: outputs <= 256 in 1..64 equal groups, of which 1..all are kept");
+    need(top >= 1 && top <= 64 && top <= keep * (N / n_groups), "moe_route_group: 1 <= top <= min(64, experts of the kept groups)");
+    auto idx = at::empty({h.size(0), top}, h.options().dtype(at::kInt));
+    auto wt = at::empty({h.size(0), top}, h.options().dtype(at::kFloat));
+    auto z = at::empty({h.size(0), N}, h.options().dtype(at::kFloat));
+    chronos::launch_hy_moe_route_group(h.data_ptr(), w.data_ptr(), z.data_ptr<float>(), idx.data_ptr<int32_t>(),
+                                       wt.data_ptr<float>(), (int)h.size(0), (int)h.size(1), (int)N, (int)top, (int)n_groups,
+                                       (int)keep, (float)scale, f32(h), stream());
+    return {idx, wt};
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(chronos, m) {
@@ -550,17 +684,26 @@ TORCH_LIBRARY_FRAGMENT(chronos, m) {
     m.def("hy_decay_pow(Tensor(a!) z, float p) -> ()");
     m.def("hy_head_norm_gate(Tensor o, Tensor src, int g_off, Tensor w, float eps, bool silu_gate, bool out_f32) -> Tensor");
     m.def("hy_window_prep(Tensor(a!) qkv, int H, int G, int D, int Dv, Tensor? v_first, Tensor? lam, Tensor pos, "
-          "Tensor tok_seq, Tensor block_table, Tensor q_norm, Tensor k_norm, float eps, Tensor? cos_sin, int dims, "
+          "Tensor tok_seq, Tensor block_table, Tensor? q_norm, Tensor? k_norm, float eps, Tensor? cos_sin, int dims, "
           "Tensor(b!) kc, Tensor(c!) vc, bool emit_v) -> Tensor");
     m.def("hy_window_attention(Tensor qkv, Tensor kc, Tensor vc, Tensor block_table, Tensor q_start, Tensor pos, "
-          "Tensor? sink, Tensor? gate, float scale, int window, int keep, int H, int max_q) -> Tensor");
+          "Tensor? sink, Tensor? gate, float scale, int window, int keep, int chunk, int H, int max_q) -> Tensor");
     m.def("hy_short_conv(Tensor x, Tensor w, Tensor tok_seq, Tensor q_start, Tensor pos0, Tensor slots, Tensor(a!) hist, "
-          "bool silu) -> Tensor");
+          "bool silu, Tensor? bias, int x_off) -> Tensor");
     m.def("hy_delta_prep(Tensor y, Tensor ab, Tensor a_log, int HK, int H, int D, float q_mul) -> (Tensor, Tensor, Tensor, Tensor)");
     m.def("hy_linear_scan(Tensor proj, int q_off, int k_off, int v_off, Tensor? qscale, Tensor? kscale, float q_mul, "
           "Tensor decay, Tensor? beta, Tensor q_start, Tensor pos0, Tensor slots, Tensor(a!) S, int HK, int H, int D, "
-          "int Dv) -> Tensor");
+          "int Dv, Tensor? vscale) -> Tensor");
     m.def("hy_moe_route_topk(Tensor h, Tensor w, Tensor bias, int top) -> (Tensor, Tensor)");
+    m.def("hy_add_rms_norm(Tensor y, Tensor(a!) x, Tensor? w_out, float eps, bool out_f32, Tensor? y2, Tensor? gate2, "
+          "Tensor? w_y, bool emit) -> Tensor");
+    m.def("hy_token_gate(Tensor a, Tensor ids, Tensor table, int col0) -> Tensor");
+    m.def("hy_ssm_prep(Tensor dt_pre, Tensor a_log) -> (Tensor, Tensor)");
+    m.def("hy_gated_group_norm(Tensor o, Tensor skip_src, int skip_off, Tensor skip_w, Tensor gate_src, int g_off, Tensor w, "
+          "int groups, float eps, bool out_f32) -> Tensor");
+    m.def("hy_rglru_scan(Tensor u, Tensor gates, Tensor sp, float c, Tensor ysrc, int y_off, Tensor q_start, Tensor pos0, "
+          "Tensor slots, Tensor(a!) S, int max_q) -> Tensor");
+    m.def("hy_moe_route_group(Tensor h, Tensor w, int top, int n_groups, int keep, float scale) -> (Tensor, Tensor)");
     m.def("hy_moe_glu_ffn(Tensor h, Tensor idx, Tensor wt, Tensor w_gu, Tensor w_down, float limit, float slope, "
           "float shift, bool tiled) -> Tensor");
 }
@@ -589,5 +732,11 @@ TORCH_LIBRARY_IMPL(chronos, CUDA, m) {
     m.impl("hy_delta_prep", &hy_delta_prep);
     m.impl("hy_linear_scan", &hy_linear_scan);
     m.impl("hy_moe_route_topk", &hy_moe_route_topk);
+    m.impl("hy_add_rms_norm", &hy_add_rms_norm);
+    m.impl("hy_token_gate", &hy_token_gate);
+    m.impl("hy_ssm_prep", &hy_ssm_prep);
+    m.impl("hy_gated_group_norm", &hy_gated_group_norm);
+    m.impl("hy_rglru_scan", &hy_rglru_scan);
+    m.impl("hy_moe_route_group", &hy_moe_route_group);
     m.impl("hy_moe_glu_ffn", &hy_moe_glu_ffn);
 }

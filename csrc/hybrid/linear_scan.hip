@@ -1,7 +1,7 @@
 // linear_scan.hip — recurrent mixers whose per-head state is a D x Dv matrix updated by rank-one writes: the gated
 // delta rule and gated linear attention, plus the short causal convolution and the per-token scalars that feed them.
 //
-//   short_conv    y[t, c] = act(sum_i w[c, i] x[t - (K-1) + i, c]) over each sequence's own tokens; inputs before the
+//   short_conv    y[t, c] = act(bias[c] + sum_i w[c, i] x[t - (K-1) + i, c]) over each sequence's own tokens; inputs before the
 //                 step's first token come from the sequence's history rows (its last K-1 inputs, by state slot), or
 //                 are zero when the step starts at position 0.  A second launch then rewrites the history.
 //   delta_prep    per token: 1 / |q|, 1 / |k| per query/key head (float), decay = exp(-exp(A) softplus(a)) and
@@ -26,14 +26,15 @@ __global__ void __launch_bounds__(256) short_conv_kernel(const T* __restrict__ x
                                                          const int32_t* __restrict__ q_start,
                                                          const int32_t* __restrict__ pos0,
                                                          const int32_t* __restrict__ slots, const T* __restrict__ hist,
-                                                         T* __restrict__ y, int C, int K, int silu) {
+                                                         T* __restrict__ y, int C, int K, int silu,
+                                                         const float* __restrict__ bias) {
     const int64_t t = blockIdx.x;
     const int b = tok_seq[t];
     const int t0 = q_start[b];
     const bool past = pos0[b] > 0;
     const T* hrow = hist + (int64_t)slots[b] * (K - 1) * C;
     for (int c = threadIdx.x; c < C; c += 256) {
-        float acc = 0.f;
+        float acc = bias != nullptr ? bias[c] : 0.f;
         for (int i = 0; i < K; ++i) {
             const int64_t s = t - (K - 1) + i;
             float v = 0.f;
@@ -111,7 +112,7 @@ template <> __device__ __forceinline__ uint16_t zero_of<uint16_t>() { return 0; 
 
 // 256 threads: wave w owns 64 / RG value columns of the workgroup's 4 x 64 / RG; a lane holds DP / RG rows of one
 // column.  LDS (floats): q [TC][DP] | k [TC][DP] | (CHD: decay rows [TC][DP]) | v [TC][64] | per token: decay, beta,
-// q scale, k scale.  The next stage's global loads are issued before the current stage's tokens are processed and
+// q scale, k scale (times the value's per-head scale when one is given).  The next stage's global loads are issued before the current stage's tokens are processed and
 // land in LDS afterwards, so the token loop never waits on global memory; the scales of q and k are folded into
 // per-token scalars (S^T k_hat = s_k S^T k, k_hat u^T = k (s_k u)^T, S^T q_hat = s_q S^T q).
 // PIPE: the one-pass token loops with LDS rows prefetched (more registers: for launches with prompt portions);
@@ -122,7 +123,7 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
         const T* __restrict__ proj, int ldp, int q_off, int k_off, int v_off, const float* __restrict__ qscale,
         const float* __restrict__ kscale, float q_mul, const float* __restrict__ decay, const float* __restrict__ beta,
         const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0, const int32_t* __restrict__ slots,
-        float* __restrict__ S, float* __restrict__ o, int HK, int H, int D, int Dv) {
+        float* __restrict__ S, float* __restrict__ o, int HK, int H, int D, int Dv, const float* __restrict__ vscale) {
     constexpr int TC = kScanTC, RG = PIPE ? kScanRGPrefill : kScanRGDecode, CW = 64 / RG, RL = DP / RG;
     constexpr int NE = TC * DP / 256, WC = 4 * CW;  // WC: value columns of the workgroup
     __shared__ __attribute__((aligned(16))) float qs[TC * DP];
@@ -174,6 +175,8 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
             sraw[1] = (DELTA && ok) ? beta[t * H + hd] : 0.f;
             sraw[2] = (qscale != nullptr && ok) ? qscale[t * HK + hk] : q_mul;
             sraw[3] = (kscale != nullptr && ok) ? kscale[t * HK + hk] : 1.f;
+            // a per-head factor on the written value u = v: k (s u)^T is all it enters (no delta correction then)
+            if (!DELTA && vscale != nullptr && ok) sraw[3] *= vscale[t * H + hd];
         }
     };
     auto land = [&]() {
@@ -327,16 +330,17 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
 
 }  // namespace hy
 
-void launch_hy_short_conv(const void* x, int ldx, const float* w, const int32_t* tok_seq, const int32_t* q_start,
-                          const int32_t* pos0, const int32_t* slots, void* hist, void* y, int T, int B, int C, int K,
-                          bool silu, bool f32, hipStream_t s) {
+// x points at the first convolved column of the first row (rows ldx apart); bias may be nullptr
+void launch_hy_short_conv(const void* x, int ldx, const float* w, const float* bias, const int32_t* tok_seq,
+                          const int32_t* q_start, const int32_t* pos0, const int32_t* slots, void* hist, void* y, int T,
+                          int B, int C, int K, bool silu, bool f32, hipStream_t s) {
     if (T == 0 || C == 0) return;
     const dim3 hg(B, (C + 255) / 256);
     if (f32) {
-        hy::short_conv_kernel<float><<<T, 256, 0, s>>>((const float*)x, ldx, w, tok_seq, q_start, pos0, slots, (const float*)hist, (float*)y, C, K, silu);
+        hy::short_conv_kernel<float><<<T, 256, 0, s>>>((const float*)x, ldx, w, tok_seq, q_start, pos0, slots, (const float*)hist, (float*)y, C, K, silu, bias);
         if (K > 1) hy::conv_hist_kernel<float><<<hg, 256, 0, s>>>((const float*)x, ldx, q_start, pos0, slots, (float*)hist, C, K);
     } else {
-        hy::short_conv_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)x, ldx, w, tok_seq, q_start, pos0, slots, (const uint16_t*)hist, (uint16_t*)y, C, K, silu);
+        hy::short_conv_kernel<uint16_t><<<T, 256, 0, s>>>((const uint16_t*)x, ldx, w, tok_seq, q_start, pos0, slots, (const uint16_t*)hist, (uint16_t*)y, C, K, silu, bias);
         if (K > 1) hy::conv_hist_kernel<uint16_t><<<hg, 256, 0, s>>>((const uint16_t*)x, ldx, q_start, pos0, slots, (uint16_t*)hist, C, K);
     }
 }
@@ -352,29 +356,29 @@ template <typename T, int DP, bool DELTA, bool CHD>
 static void linear_scan_launch(bool pipe, const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                                const float* kscale, float q_mul, const float* decay, const float* beta,
                                const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
-                               int HK, int H, int D, int Dv, hipStream_t s) {
+                               int HK, int H, int D, int Dv, const float* vscale, hipStream_t s) {
     constexpr bool HAS_PIPE = DELTA != CHD;   // the two combinations with a pipelined token loop
     if constexpr (HAS_PIPE) {
         if (pipe) {
             const dim3 grid(B, H, (Dv + 4 * (64 / hy::kScanRGPrefill) - 1) / (4 * (64 / hy::kScanRGPrefill)));
             hy::linear_scan_kernel<T, DP, DELTA, CHD, true><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
-                                                                                beta, q_start, pos0, slots, S, o, HK, H, D, Dv);
+                                                                                beta, q_start, pos0, slots, S, o, HK, H, D, Dv, vscale);
             return;
         }
     }
     const dim3 grid(B, H, (Dv + 4 * (64 / hy::kScanRGDecode) - 1) / (4 * (64 / hy::kScanRGDecode)));
     hy::linear_scan_kernel<T, DP, DELTA, CHD, false><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
-                                                                         beta, q_start, pos0, slots, S, o, HK, H, D, Dv);
+                                                                         beta, q_start, pos0, slots, S, o, HK, H, D, Dv, vscale);
 }
 
 template <typename T, bool DELTA, bool CHD>
 static bool linear_scan_d(bool pipe, const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                           const float* kscale, float q_mul, const float* decay, const float* beta, const int32_t* q_start,
                           const int32_t* pos0, const int32_t* slots, float* S, float* o, int B, int HK, int H, int D,
-                          int Dv, hipStream_t s) {
+                          int Dv, const float* vscale, hipStream_t s) {
 #define HY_LS(DP)                                                                                                     \
     linear_scan_launch<T, DP, DELTA, CHD>(pipe, proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, \
-                                          pos0, slots, S, o, B, HK, H, D, Dv, s)
+                                          pos0, slots, S, o, B, HK, H, D, Dv, vscale, s)
     if (D <= 32) HY_LS(32);
     else if (D <= 64) HY_LS(64);
     else if (D <= 128) HY_LS(128);
@@ -384,18 +388,18 @@ static bool linear_scan_d(bool pipe, const T* proj, int ldp, int q_off, int k_of
     return true;
 }
 
-// delta: beta != nullptr.  chd: decay holds one number per state row ([T, H, D]) instead of one per head ([T, H]).
+// delta: beta != nullptr.  vscale (float [T, H], may be nullptr; without delta only): a factor on the written value.  chd: decay holds one number per state row ([T, H, D]) instead of one per head ([T, H]).
 // Returns false when D has no instantiation (D > 256).
 bool launch_hy_linear_scan(const void* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                            const float* kscale, float q_mul, const float* decay, bool chd, const float* beta,
                            const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int T,
-                           int B, int HK, int H, int D, int Dv, bool f32, hipStream_t s) {
+                           int B, int HK, int H, int D, int Dv, const float* vscale, bool f32, hipStream_t s) {
     if (B == 0) return true;
     const bool pipe = T > B;   // some sequence brings more than one token
     const bool delta = beta != nullptr;
 #define HY_LSD(T, DELTA, CHD)                                                                                        \
     return linear_scan_d<T, DELTA, CHD>(pipe, (const T*)proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, \
-                                        q_start, pos0, slots, S, o, B, HK, H, D, Dv, s)
+                                        q_start, pos0, slots, S, o, B, HK, H, D, Dv, vscale, s)
     if (f32) {
         if (delta && chd) HY_LSD(float, true, true);
         if (delta) HY_LSD(float, true, false);

@@ -4,6 +4,9 @@
 //           hybrid_elementwise.hip), then one wave per token: softmax over all N, the `top` largest
 //           of score + correction chosen (the correction steers the choice only), weights = the chosen outputs' plain
 //           scores, not renormalised.  Ties go to the lower index.
+//   route_group  sigmoid scores; the outputs form equal groups of neighbours, a group scores the sum of its two
+//           largest scores, only the best `keep` groups stay eligible, the `top` largest eligible scores are chosen and
+//           weighted by score / (sum of the chosen + 1e-20) * scale.
 //   ffn     per token: sum over its chosen experts of weight * W_down act(W_up h); an index >= E is an identity
 //           expert (weight * h).  Token-parallel form: one workgroup per token streams the chosen experts' weights
 //           (the decode regime: few tokens, every expert matrix read about once; float accumulation throughout).
@@ -166,6 +169,81 @@ __global__ void __launch_bounds__(256) moe_select_topk_kernel(const float* __res
     if (lane < top) wt[t * top + lane] = mine / sum;
 }
 
+// One wave per token: sigmoid scores of z [T, N], the choice limited to the best groups (ng groups of N / ng
+// neighbouring outputs, a group's score = the sum of its two largest scores, the `keep` best stay; ties: the lower
+// index), then the `top` largest eligible scores (ties: the lower index), weights = score / (their sum + 1e-20) * scale.
+// ng <= 64 (lane g ranks group g), top <= 64 (lane k keeps the k-th choice).  LDS per wave: N scores, ng flags.
+__global__ void __launch_bounds__(256) moe_select_group_kernel(const float* __restrict__ z, int32_t* __restrict__ idx,
+                                                               float* __restrict__ wt, int rows, int N, int top, int ng,
+                                                               int keep, float scale) {
+    __shared__ float sc[4][256];
+    __shared__ int okg[4][64];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int64_t t = (int64_t)blockIdx.x * 4 + wv;
+    if (t >= rows) return;   // (a whole wave leaves; the waves of a block share no barrier)
+    const int per = N / ng;
+    float s[4], c[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        s[j] = e < N ? sigmoidf_(z[t * N + e]) : 0.f;
+        if (e < N) sc[wv][e] = s[j];
+    }
+    // (wave-private LDS rows: a wave's own writes are visible to its later reads)
+    if (keep < ng) {
+        float gsc = -INFINITY;
+        if (lane < ng) {
+            float a = -INFINITY, b = -INFINITY;   // the group's two largest
+            for (int i = 0; i < per; ++i) {
+                const float v = sc[wv][lane * per + i];
+                if (v > a) { b = a; a = v; }
+                else if (v > b) b = v;
+            }
+            gsc = per > 1 ? a + b : a;
+        }
+        int rank = 0;   // groups that come before this one
+        for (int g = 0; g < ng; ++g) {
+            const float o = __shfl(gsc, g, 64);
+            rank += (o > gsc || (o == gsc && g < lane)) ? 1 : 0;
+        }
+        if (lane < ng) okg[wv][lane] = rank < keep ? 1 : 0;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int e = lane + 64 * j;
+        c[j] = (e < N && (keep >= ng || okg[wv][e / per])) ? s[j] : -INFINITY;
+    }
+    float sum = 0.f, mine = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float bv = -INFINITY;
+        int be = 0x7fffffff;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int e = lane + 64 * j;
+            if (e < N && (c[j] > bv || (c[j] == bv && e < be && c[j] != -INFINITY))) {
+                bv = c[j]; be = e;
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float ov = __shfl_xor(bv, o, 64);
+            const int oe = __shfl_xor(be, o, 64);
+            if (ov > bv || (ov == bv && oe < be)) {
+                bv = ov; be = oe;
+            }
+        }
+        sum += bv;
+        if (k == lane) {
+            mine = bv;
+            idx[t * top + k] = be;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (lane + 64 * j == be) c[j] = -INFINITY;
+    }
+    if (lane < top) wt[t * top + lane] = mine / (sum + 1e-20f) * scale;
+}
+
 // Gated experts: per token sum_k weight_k * W_down,e ( g sigmoid(slope g) (u + shift) ), g = min(W_gate,e h, limit),
 // u = clamp(W_up,e h, +-limit).  w_gu [E, 2F, d]: gate rows then up rows, or (tiled) in the grouped path's tile order.
 // LDS: h (d) | gate, up (2F) | out (d).
@@ -255,6 +333,14 @@ void launch_hy_moe_route_topk(const void* h, const void* w, const float* bias, f
     if (T == 0) return;
     launch_hy_rowdot(h, w, bias, z, T, d, N, f32, s);
     hy::moe_select_topk_kernel<<<(T + 3) / 4, 256, 0, s>>>(z, idx, wt, T, N, top);
+}
+
+// z: float [T, N] scratch for the router logits, N <= 256, groups <= 64, top <= 64
+void launch_hy_moe_route_group(const void* h, const void* w, float* z, int32_t* idx, float* wt, int T, int d, int N,
+                               int top, int ng, int keep, float scale, bool f32, hipStream_t s) {
+    if (T == 0) return;
+    launch_hy_rowdot(h, w, nullptr, z, T, d, N, f32, s);
+    hy::moe_select_group_kernel<<<(T + 3) / 4, 256, 0, s>>>(z, idx, wt, T, N, top, ng, keep, scale);
 }
 
 void launch_hy_moe_glu_token(const void* h, const int32_t* idx, const float* wt, const void* w_gu, const void* w_down,

@@ -1,7 +1,7 @@
 // window_attention.hip — grouped-query softmax attention over paged keys and values through a sliding window that
 // also keeps each sequence's first tokens, with a learned sink per head in the softmax denominator.
 //
-//   window_prep       per token: per-head RMS norm (float) and rotation (cos / sin from a float table made in double
+//   window_prep       per token: per-head RMS norm (float; skipped when no norm weights are given) and rotation (cos / sin from a float table made in double
 //                     precision) of the query heads (in place) and key heads; the values optionally mixed with the
 //                     same token's values of an earlier layer, (1 - lam) v + lam v_first; keys and values written to
 //                     the token's page and slot of kc [NB, BS, G, D] / vc [NB, BS, G, Dv].
@@ -12,7 +12,11 @@
 //                     accumulation, online softmax in float) and value columns for the output.  The key range of a
 //                     tile of queries is [0, keep_first) and [first query - window + 1, last query]; tiles of keys
 //                     between the two are never touched, and each row masks by its own position:
-//                         visible(i, j) = j <= i and (window == 0 or i - j < window or j < keep_first).
+//                         visible(i, j) = j <= i and (window == 0 or i - j < window or j < keep_first)
+//                                         and (chunk == 0 or j >= floor(i / chunk) * chunk).
+//                     With chunk > 0 a query sees only the keys of its own chunk of positions (counted from the
+//                     sequence's position 0, wherever a prompt was cut); the tile walk starts at the first query's
+//                     chunk start.
 //                     After the last key the sink joins the denominator: l += exp(sink_h - m) (no value), and the
 //                     row is multiplied by sigmoid(gate) when a gate is given.
 // Prompt portions, decode rows and mixed steps are one code path (a decode row is a tile of one token).
@@ -43,20 +47,22 @@ __global__ void __launch_bounds__(256) window_prep_kernel(
     for (int j = wv; j < H + G; j += 4) {  // heads 0..H-1: queries (in place); H..H+G-1: keys (to the cache)
         const T* src = base + (int64_t)j * D;
         const float* nw = j < H ? q_norm : k_norm;
+        if (nw == nullptr && dims == 0 && j < H) continue;  // plain queries stay as the projection wrote them
         float ss = 0.f;
         for (int i = lane; i < D; i += 64) {
             const float v = ld<T>(src + i);
             row[i] = v;
             ss += v * v;
         }
-        const float inv = 1.f / sqrtf(wave_sum(ss) / (float)D + eps);
+        const float inv = nw != nullptr ? 1.f / sqrtf(wave_sum(ss) / (float)D + eps) : 1.f;
         T* dst = j < H ? base + (int64_t)j * D : kc + (slot * G + (j - H)) * D;
         // (wave-private LDS row: the wave's own writes above are visible to its reads below without a barrier,
         // the compiler orders LDS accesses of one wave)
         for (int i = lane; i < D; i += 64) {
-            float v = row[i] * inv * nw[i];
-            if (i < half) v = v * cs[i] - row[i + half] * inv * nw[i + half] * cs[half + i];
-            else if (i < dims) v = v * cs[i - half] + row[i - half] * inv * nw[i - half] * cs[i];
+            auto nrm = [&](int c) { return nw != nullptr ? row[c] * inv * nw[c] : row[c]; };
+            float v = nrm(i);
+            if (i < half) v = v * cs[i] - nrm(i + half) * cs[half + i];
+            else if (i < dims) v = v * cs[i - half] + nrm(i - half) * cs[i];
             st<T>(dst + i, v);
         }
     }
@@ -85,7 +91,7 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
         const T* __restrict__ qkv, int ldq, const T* __restrict__ kc, const T* __restrict__ vc,
         const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ q_start,
         const int32_t* __restrict__ pos, const float* __restrict__ sink, const float* __restrict__ gate,
-        T* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int QT,
+        T* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int chunk, int QT,
         int rows_cap) {
     extern __shared__ __attribute__((aligned(16))) unsigned char wa_smem[];
     constexpr int PAD = WaPad<T>::V;
@@ -108,7 +114,8 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
     }
     const int p_lo = pos[t0], p_hi = pos[t1 - 1];
     // tokens of a range sit at consecutive positions, so the tile's queries are p_lo .. p_hi
-    const int w_lo = window > 0 ? max(0, p_lo - window + 1) : 0;
+    // the first key any row of the tile may see (the bounds of both masks grow with the position)
+    const int w_lo = max(window > 0 ? max(0, p_lo - window + 1) : 0, chunk > 0 ? p_lo / chunk * chunk : 0);
     const int w_start = w_lo / kWaKT * kWaKT;
     // kept first tokens below the window's first tile: keys [0, k_end) (those from w_start on pass the window tiles'
     // own test), so no key is ever counted twice
@@ -165,7 +172,8 @@ __global__ void __launch_bounds__(256) window_attention_kernel(
             for (int r = 0; r < kWaRB; ++r) {
                 const int rr = min(r0 + r, rows - 1);
                 const int pi = p_lo + rr / R;
-                const bool vis = j < j_end && j <= pi && (window <= 0 || pi - j < window || j < keep);
+                const bool vis = j < j_end && j <= pi && (window <= 0 || pi - j < window || j < keep) &&
+                                 (chunk <= 0 || j >= pi / chunk * chunk);
                 const float sv = vis ? s[r] * scale : -INFINITY;
                 const float mn = fmaxf(m_[q][r], wave_max(sv));
                 const float pw = mn == -INFINITY ? 0.f : expf(sv - mn);
@@ -251,19 +259,19 @@ int hy_window_rows_cap(int R, int D, int Dv, bool f32) {
 
 bool launch_hy_window_attention_mfma(const uint16_t*, int, const uint16_t*, const uint16_t*, const int32_t*, int,
                                      const int32_t*, const int32_t*, const float*, const float*, uint16_t*, int, int, int,
-                                     int, int, int, int, float, int, int, int, float*, float*, int64_t, hipStream_t);
+                                     int, int, int, int, float, int, int, int, int, float*, float*, int64_t, hipStream_t);
 
 // bfloat16 at matrix-core sizes runs window_attention_mfma.hip; float32 and every other size the general kernel.
 void launch_hy_window_attention(const void* qkv, int ld, const void* kc, const void* vc, const int32_t* block_table,
                                 int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
                                 const float* gate, void* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
-                                float scale, int window, int keep, bool f32, int nsplit, float* part_o, float* part_ml,
-                                int64_t total_rows, hipStream_t s) {
+                                float scale, int window, int keep, int chunk, bool f32, int nsplit, float* part_o,
+                                float* part_ml, int64_t total_rows, hipStream_t s) {
     if (B == 0 || max_q == 0) return;
     if (!f32 && launch_hy_window_attention_mfma((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc,
                                                 block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, B,
-                                                max_q, H, G, D, Dv, BS, scale, window, keep, nsplit, part_o, part_ml,
-                                                total_rows, s))
+                                                max_q, H, G, D, Dv, BS, scale, window, keep, chunk, nsplit, part_o,
+                                                part_ml, total_rows, s))
         return;
     const int R = H / G;   // the caller has checked R <= 64, Dv <= 256 and that hy_window_rows_cap is not 0
     const int rows_cap = hy_window_rows_cap(R, D, Dv, f32);
@@ -273,11 +281,11 @@ void launch_hy_window_attention(const void* qkv, int ld, const void* kc, const v
     if (f32) {
         auto kern = hy::window_attention_kernel<float>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<grid, 256, bytes, s>>>((const float*)qkv, ld, (const float*)kc, (const float*)vc, block_table, max_blocks, q_start, pos, sink, gate, (float*)out, H, G, D, Dv, BS, scale, window, keep, QT, rows_cap);
+        kern<<<grid, 256, bytes, s>>>((const float*)qkv, ld, (const float*)kc, (const float*)vc, block_table, max_blocks, q_start, pos, sink, gate, (float*)out, H, G, D, Dv, BS, scale, window, keep, chunk, QT, rows_cap);
     } else {
         auto kern = hy::window_attention_kernel<uint16_t>;
         (void)hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
-        kern<<<grid, 256, bytes, s>>>((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc, block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, H, G, D, Dv, BS, scale, window, keep, QT, rows_cap);
+        kern<<<grid, 256, bytes, s>>>((const uint16_t*)qkv, ld, (const uint16_t*)kc, (const uint16_t*)vc, block_table, max_blocks, q_start, pos, sink, gate, (uint16_t*)out, H, G, D, Dv, BS, scale, window, keep, chunk, QT, rows_cap);
     }
 }
 

@@ -17,6 +17,7 @@
 //     as two bfloat16 terms (rounded value + remainder), which keeps the float softmax weights nearly exact.
 // After the last tile the head's sink joins the denominator and the row is scaled by sigmoid(gate).  Launches of few
 // rows (decode) deal a row block's key tiles to several workgroups and merge the float partials in a second kernel.
+// With chunk > 0 a row also hides the keys below its own chunk of positions (key >= floor(pos / chunk) * chunk).
 // Sizes: D % 32 == 0, Dv % 16 == 0, D <= 256, Dv <= 256.  Everything else takes the general kernel.
 #include <algorithm>
 
@@ -32,8 +33,8 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
         const uint16_t* __restrict__ qkv, int ldq, const uint16_t* __restrict__ kc, const uint16_t* __restrict__ vc,
         const int32_t* __restrict__ block_table, int max_blocks, const int32_t* __restrict__ q_start,
         const int32_t* __restrict__ pos, const float* __restrict__ sink, const float* __restrict__ gate,
-        uint16_t* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int nsplit,
-        float* __restrict__ part_o, float* __restrict__ part_ml) {
+        uint16_t* __restrict__ out, int H, int G, int D, int Dv, int BS, float scale, int window, int keep, int chunk,
+        int nsplit, float* __restrict__ part_o, float* __restrict__ part_ml) {
     extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
     constexpr int KT = WKT, NT = 64 * NW, RPB = 16 * NW, PP = KT / 2;
     const int R = H / G;
@@ -69,8 +70,11 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
     const float scale2 = scale * 1.4426950408889634f;
     const int32_t* bt = block_table + (int64_t)b * max_blocks;
     const int kchunks = D / 8, vchunks = Dv / 8;
-    const int w_lo = window > 0 ? max(0, pmin - window + 1) : 0;
+    // the first key any row of the block may see: the window's or the chunk's lower bound of the first row
+    const int w_lo = max(window > 0 ? max(0, pmin - window + 1) : 0, chunk > 0 ? pmin / chunk * chunk : 0);
     const int w_start = w_lo / KT * KT;
+    const int c_lo = chunk > 0 ? prow / chunk * chunk : 0;        // this row's chunk starts here
+    const int c_lo_max = chunk > 0 ? pmax / chunk * chunk : 0;    // the last row's
     // kept first tokens below the window's first tile are keys [0, k_end); those from w_start on pass the window
     // tiles' own test, so no key is counted twice
     const int k_end = window > 0 ? min(keep, w_start) : 0;
@@ -119,7 +123,8 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
         // scores, maxima and sums live in the base-2 domain (score * scale * log2 e): one multiply and one
         // subtraction in front of the hardware's exp2.  A tile that every row of the block sees whole (the common case
         // inside a window) skips the per-key visibility tests.
-        const bool whole = k0 + KT - 1 <= min(k_last, pmin) && (window <= 0 || kept || pmax - k0 < window);
+        const bool whole = k0 + KT - 1 <= min(k_last, pmin) && (window <= 0 || kept || pmax - k0 < window) &&
+                           k0 >= c_lo_max;
         float mx = -INFINITY;
         if (whole) {
 #pragma unroll
@@ -135,7 +140,8 @@ __global__ void __launch_bounds__(64 * NW) window_attention_mfma_kernel(
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int key = k0 + 16 * kt + 4 * g4 + i;
-                    const bool vis = key <= k_last && key <= prow && (window <= 0 || prow - key < window || key < keep);
+                    const bool vis = key <= k_last && key <= prow && (window <= 0 || prow - key < window || key < keep) &&
+                                     key >= c_lo;
                     const float sv = vis ? S[kt][i] * scale2 : -INFINITY;
                     S[kt][i] = sv;
                     mx = fmaxf(mx, sv);
@@ -255,7 +261,8 @@ template <int NS, int NCT, int NW>
 static void wa_mfma_launch(const uint16_t* qkv, int ldq, const uint16_t* kc, const uint16_t* vc, const int32_t* bt,
                            int max_blocks, const int32_t* q_start, const int32_t* pos, const float* sink,
                            const float* gate, uint16_t* out, int B, int max_q, int H, int G, int D, int Dv, int BS,
-                           float scale, int window, int keep, int nsplit, float* part_o, float* part_ml, hipStream_t s) {
+                           float scale, int window, int keep, int chunk, int nsplit, float* part_o, float* part_ml,
+                           hipStream_t s) {
     auto kern = hy::window_attention_mfma_kernel<NS, NCT, NW>;
     const int bytes = hy::WKT * (D * 2 + 16) + Dv * (hy::WKT * 2 + 8);
     static int set_bytes = 0;
@@ -265,7 +272,7 @@ static void wa_mfma_launch(const uint16_t* qkv, int ldq, const uint16_t* kc, con
     }
     const dim3 grid(B, (max_q * (H / G) + 16 * NW - 1) / (16 * NW) * nsplit, G);
     kern<<<grid, 64 * NW, bytes, s>>>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, H, G, D, Dv, BS, scale,
-                                      window, keep, nsplit, part_o, part_ml);
+                                      window, keep, chunk, nsplit, part_o, part_ml);
 }
 
 bool hy_window_mfma_ok(int ldq, int D, int Dv) { return !(D % 32 || Dv % 16 || D > 256 || Dv > 256 || ldq % 8); }
@@ -274,12 +281,14 @@ bool hy_window_mfma_ok(int ldq, int D, int Dv) { return !(D % 32 || Dv % 16 || D
 // of the chip idle — decode rows, a lone short portion: enough workgroups to cover the CUs four times, at least 2 key
 // tiles per split, at most 16.  The tile count follows from sizes the host knows (the window, or the block table's
 // width when there is none).  1 for float32 and sizes the matrix-core kernel does not serve.
-int hy_window_nsplit(bool f32, int ldq, int B, int max_q, int H, int G, int D, int Dv, int window, int keep, int max_ctx) {
+int hy_window_nsplit(bool f32, int ldq, int B, int max_q, int H, int G, int D, int Dv, int window, int keep, int chunk,
+                     int max_ctx) {
     if (f32 || !hy_window_mfma_ok(ldq, D, Dv) || B <= 0) return 1;
     const int rows = max_q * (H / G);
     const int wgs = B * ((rows + (rows > 64 ? 127 : 63)) / (rows > 64 ? 128 : 64)) * G;
     if (wgs >= 512) return 1;
-    const int span = window > 0 ? std::min(max_ctx, window + max_q) : max_ctx;
+    int span = window > 0 ? std::min(max_ctx, window + max_q) : max_ctx;
+    if (chunk > 0) span = std::min(span, chunk + max_q);   // a row block's keys start in its first row's chunk
     const int tiles = span / hy::WKT + 1 + (window > 0 ? (std::min(keep, max_ctx) + hy::WKT - 1) / hy::WKT : 0);
     int want = (1024 + wgs - 1) / wgs;
     want = std::min(want, std::min(16, tiles / 2));
@@ -291,11 +300,11 @@ int hy_window_nsplit(bool f32, int ldq, int B, int max_q, int H, int G, int D, i
 bool launch_hy_window_attention_mfma(const uint16_t* qkv, int ldq, const uint16_t* kc, const uint16_t* vc,
                                      const int32_t* bt, int max_blocks, const int32_t* q_start, const int32_t* pos,
                                      const float* sink, const float* gate, uint16_t* out, int B, int max_q, int H, int G,
-                                     int D, int Dv, int BS, float scale, int window, int keep, int nsplit, float* part_o,
-                                     float* part_ml, int64_t total_rows, hipStream_t s) {
+                                     int D, int Dv, int BS, float scale, int window, int keep, int chunk, int nsplit,
+                                     float* part_o, float* part_ml, int64_t total_rows, hipStream_t s) {
     if (!hy_window_mfma_ok(ldq, D, Dv)) return false;
     if (B == 0 || max_q == 0) return true;
-#define HY_WAM(NS, NCT, NW) wa_mfma_launch<NS, NCT, NW>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, B, max_q, H, G, D, Dv, BS, scale, window, keep, nsplit, part_o, part_ml, s)
+#define HY_WAM(NS, NCT, NW) wa_mfma_launch<NS, NCT, NW>(qkv, ldq, kc, vc, bt, max_blocks, q_start, pos, sink, gate, out, B, max_q, H, G, D, Dv, BS, scale, window, keep, chunk, nsplit, part_o, part_ml, s)
     // 8 waves per workgroup when a sequence brings more than 64 rows per key/value head: a staged tile then serves
     // 128 rows and every SIMD holds two waves
     const bool nw8 = max_q * (H / G) > 64;

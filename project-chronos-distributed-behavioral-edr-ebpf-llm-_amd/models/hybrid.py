@@ -1,8 +1,10 @@
 """Hybrid decoders: a list of layers, each with a token mixer of some kind (recurrent matrix memory, latent
-attention, windowed attention with sinks, gated delta rule, gated linear attention) and an optional feed-forward
-(dense, gated, mixture of experts), on a float32 residual stream.  The stream's rule is a parameter of the
-configuration: the norm on the sublayer's OUTPUT (``out_norm``: x <- x + layer_norm(sublayer(x))) or AFTER the sum
-(``post_norm``: x <- rms_norm(alpha x + sublayer(x))).
+attention, windowed or chunked attention, gated delta rule, gated linear attention, state-space duality, real-gated
+linear recurrence) and an optional feed-forward (dense, gated, mixture of experts), on a float32 residual stream.
+The stream's rule is a parameter of the configuration: the norm on the sublayer's OUTPUT (``out_norm``:
+x <- x + layer_norm(sublayer(x))), AFTER the sum (``post_norm``: x <- rms_norm(alpha x + sublayer(x))) or on the
+sublayer's INPUT (``pre_norm``: x <- x + sublayer(rms_norm(x))).  A range of layers may run several times in a row
+with the same weights (``loop``); every run has its own pages and state.
 
 This module is the design-independent part: the mixer and feed-forward kinds with their sizes and constants as
 parameters, the cache that holds pages for the attention layers and state slots for the recurrent ones, and the
@@ -89,11 +91,17 @@ class WindowAttentionSpec:
     rope_scaling: Optional[tuple] = None
     v_mix: bool = False
     v_mix_first: bool = False  # this layer is the source of the mixed-in values (and does not mix itself)
+    chunk: int = 0           # > 0: a query sees only the keys of its own chunk of this many positions
+    qk_norm: bool = True     # per-head RMS norm of queries and keys
+    sink: bool = True        # a learned softmax sink per head
+    gate: bool = True        # a sigmoid output gate per head
+    bias: bool = False       # the q, k, v projections add a bias
     kind: str = "window_attention"
 
     def params(self, d: int) -> int:
-        return d * (self.heads * self.dim + self.kv_heads * (self.dim + self.vdim) + self.heads) + 2 * self.dim + \
-            self.heads + 1 + self.heads * self.vdim * d
+        qkv = self.heads * self.dim + self.kv_heads * (self.dim + self.vdim)
+        return d * (qkv + self.heads * self.gate) + 2 * self.dim * self.qk_norm + self.heads * self.sink + 1 + \
+            self.heads * self.vdim * d + qkv * self.bias
 
 
 @dataclass
@@ -129,6 +137,49 @@ class GLASpec:
 
 
 @dataclass
+class Mamba2Spec:
+    """State-space duality: per head a state x vdim matrix S <- exp(-exp(A) dt) S + dt B x^T, read by C, with B and C
+    shared by the heads of a group; x, B and C pass a short causal convolution (with bias) and SiLU; the read-out
+    plus D x is gated by silu(z) and then RMS-normed in ``norm_groups`` equal parts."""
+    heads: int
+    vdim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int = 1
+    kind: str = "mamba2"
+
+    @property
+    def inner(self) -> int:
+        return self.heads * self.vdim
+
+    @property
+    def conv_channels(self) -> int:
+        return self.inner + 2 * self.groups * self.state
+
+    def params(self, d: int) -> int:
+        return d * (2 * self.inner + 2 * self.groups * self.state + self.heads) + self.conv_channels * (self.conv + 1) + \
+            3 * self.heads + self.inner + self.inner * d
+
+
+@dataclass
+class RGLRUSpec:
+    """Real-gated linear recurrent unit: per channel S <- a S + sqrt(1 - a^2) i u with a = exp(-c r softplus(lam)),
+    the gates r and i sigmoids of block-diagonal projections of u, u a short causal convolution (with bias) of one
+    input branch; the other branch, through gelu, multiplies the state on the way out."""
+    width: int
+    blocks: int
+    conv: int
+    c: float = 8.0
+    kind: str = "rglru"
+
+    def params(self, d: int) -> int:
+        bw = self.width // self.blocks
+        return 2 * self.width * (d + 1) + self.width * (self.conv + 1) + 2 * self.blocks * bw * (bw + 1) + self.width + \
+            self.width * d
+
+
+@dataclass
 class GluFFSpec:
     """Gated feed-forward: y = g sigmoid(slope g) (u + shift) with g = min(W_gate h, limit) and
     u = clamp(W_up h, -limit, limit)."""
@@ -153,6 +204,24 @@ class MoEGluSpec:
 
 
 @dataclass
+class MoEGroupGluSpec:
+    """Mixture of gated experts behind a sigmoid router whose choice is limited to the best groups of neighbouring
+    experts (a group scores the sum of its two largest scores); weights = chosen scores / their sum * scale.  With
+    ``shared_ff`` > 0 a shared gated expert of that size runs for every token, times sigmoid of one more projection."""
+    experts: int
+    top: int
+    ff: int
+    groups: int = 1
+    keep: int = 1
+    scale: float = 1.0
+    shared_ff: int = 0
+    limit: float = float("inf")   # the gated unit without clamp: silu(g) u
+    slope: float = 1.0
+    shift: float = 0.0
+    kind: str = "moe_group_glu"
+
+
+@dataclass
 class LayerSpec:
     mixer: object
     ff: Optional[object]
@@ -168,13 +237,26 @@ class HybridConfig:
     logit_scale: float = 1.0
     max_position: int = 8192
     architecture: str = "hybrid"
-    residual: str = "out_norm"     # "out_norm": x <- x + layer_norm(y);  "post_norm": x <- rms_norm(alpha x + y)
+    residual: str = "out_norm"     # "out_norm": x <- x + layer_norm(y);  "post_norm": x <- rms_norm(alpha x + y);
+    #                                "pre_norm": x <- x + sublayer(rms_norm(x))
     residual_alpha: float = 1.0
     tied_head: bool = False        # the logits come from the embedding table
+    loop: Optional[tuple] = None   # (start, stop, times): layers start .. stop-1 run ``times`` times in a row
+    token_side: int = 0            # > 0: after every layer's feed-forward a gated, RMS-normed projection of this many
+    #                                columns of a second embedding table (layer i owns columns [i dim, (i+1) dim))
 
     @property
     def num_layers(self) -> int:
-        return len(self.layers)
+        return len(self.runs)
+
+    @property
+    def runs(self) -> list:
+        """Layer index of every layer run, in order (the looped range repeated); pages and state are per run."""
+        n = len(self.layers)
+        if not self.loop or self.loop[2] <= 1:
+            return list(range(n))
+        a, b, t = self.loop
+        return list(range(a)) + list(range(a, b)) * t + list(range(b, n))
 
     def param_count(self) -> int:
         d = self.hidden_size
@@ -193,7 +275,11 @@ class HybridConfig:
                 f = l.ff
                 n += d + {"dense": lambda: 2 * d * f.ff, "glu": lambda: 3 * d * f.ff,
                           "moe": lambda: f.experts * 2 * d * f.ff + (f.experts + f.identity) * (d + 1),
-                          "moe_glu": lambda: f.experts * (3 * d * f.ff + d + 1)}[f.kind]()
+                          "moe_glu": lambda: f.experts * (3 * d * f.ff + d + 1),
+                          "moe_group_glu": lambda: f.experts * (3 * d * f.ff + d) + (
+                              3 * d * f.shared_ff + d if f.shared_ff else 0)}[f.kind]()
+            if self.token_side:
+                n += self.token_side * (2 * d + self.vocab_size) + d
         return n
 
 
@@ -203,12 +289,13 @@ class HybridConfig:
 
 
 class HybridCache:
-    """Per latent-attention layer a paged latent cache [NB, BS, kv_rank + rot_dim], per windowed-attention layer
+    """Per latent-attention layer run a paged latent cache [NB, BS, kv_rank + rot_dim], per windowed-attention run
     paged keys [NB, BS, G, D] and values [NB, BS, G, Dv], all in the activation dtype (block 0 is the engine's scratch
-    block); per recurrent layer float32 state rows S [NS, H, D, Dv] (the matrix-memory layers also n [NS, H, D] and
-    m [NS, H]; the delta-rule layers also the last conv - 1 inputs of their convolution, ``hist`` [NS, conv - 1, C] in
-    the activation dtype), one row per engine slot plus a scratch row (``scratch_slot``) for the decode rows of slots
-    that hold no running sequence.
+    block); per recurrent run float32 state rows S [NS, H, D, Dv] (the matrix-memory layers also n [NS, H, D] and
+    m [NS, H]; the gated linear recurrence keeps S [NS, width]; layers with a short convolution also its last
+    conv - 1 inputs, ``hist`` [NS, conv - 1, C] in the activation dtype), one row per engine slot plus a scratch row
+    (``scratch_slot``) for the decode rows of slots that hold no running sequence.  Tensors are keyed by the index of
+    the layer RUN: a layer inside a loop has one set per pass.
 
     A sequence's state needs no reset: a step whose first token sits at position 0 starts from zero."""
 
@@ -223,7 +310,7 @@ class HybridCache:
         self.kc: dict[int, torch.Tensor] = {}
         self.vc: dict[int, torch.Tensor] = {}
         self.hist: dict[int, torch.Tensor] = {}
-        for li, l in enumerate(cfg.layers):
+        for li, l in enumerate(cfg.layers[i] for i in cfg.runs):
             mx = l.mixer
             if mx.kind == "latent_attention":
                 self.lat[li] = torch.zeros(num_blocks, block_size, mx.kv_rank + mx.rot_dim, device=device,
@@ -242,12 +329,19 @@ class HybridCache:
                 if mx.kind == "delta_rule":
                     ch = 2 * mx.kv_heads * mx.dim + mx.heads * mx.vdim
                     self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), ch, device=device, dtype=act_dtype)
+            elif mx.kind == "mamba2":
+                self.S[li] = torch.zeros(slots + 1, mx.heads, mx.state, mx.vdim, device=device, dtype=torch.float32)
+                self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), mx.conv_channels, device=device,
+                                            dtype=act_dtype)
+            elif mx.kind == "rglru":
+                self.S[li] = torch.zeros(slots + 1, mx.width, device=device, dtype=torch.float32)
+                self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), mx.width, device=device, dtype=act_dtype)
 
     @staticmethod
     def bytes_per_block(cfg: HybridConfig, block_size: int, act_dtype) -> int:
         eb = 4 if act_dtype == torch.float32 else 2
         per_token = 0
-        for l in cfg.layers:
+        for l in (cfg.layers[i] for i in cfg.runs):
             m = l.mixer
             if m.kind == "latent_attention":
                 per_token += m.kv_rank + m.rot_dim
@@ -272,6 +366,7 @@ class HybridLayerWeights:
     mix: dict
     norm2: Optional[torch.Tensor] = None
     ff: dict = field(default_factory=dict)
+    side: dict = field(default_factory=dict)   # the per-layer token input: w_gate, w_proj, norm, col0
 
 
 @dataclass
@@ -280,13 +375,15 @@ class HybridWeights:
     layers: list
     final_norm: torch.Tensor
     head: torch.Tensor
+    side_embed: Optional[torch.Tensor] = None
 
     def nbytes(self) -> int:
         n = 0
-        for t in (self.embed, self.final_norm, self.head):
-            n += t.numel() * t.element_size()
+        for t in (self.embed, self.final_norm, self.head, self.side_embed):
+            if t is not None:
+                n += t.numel() * t.element_size()
         for l in self.layers:
-            for t in (l.norm1, l.norm2, *l.mix.values(), *l.ff.values()):
+            for t in (l.norm1, l.norm2, *l.mix.values(), *l.ff.values(), *l.side.values()):
                 if isinstance(t, torch.Tensor):
                     n += t.numel() * t.element_size()
         return n
@@ -330,11 +427,40 @@ def pack_window_attention(spec: WindowAttentionSpec, t: dict, device, act_dtype)
     the per-head gate rows are a few-row float32-output projection."""
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
     f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
-    out = dict(w_qkv=a(torch.cat([t["q"], t["k"], t["v"]], 0)), q_norm=f(t["q.norm"]), k_norm=f(t["k.norm"]),
-               sink=f(t["sink"]), w_g=a(t["g"]), w_o=a(t["o"]))
+    out = dict(w_qkv=a(torch.cat([t["q"], t["k"], t["v"]], 0)), w_o=a(t["o"]))
+    if spec.qk_norm:
+        out.update(q_norm=f(t["q.norm"]), k_norm=f(t["k.norm"]))
+    if spec.sink:
+        out["sink"] = f(t["sink"])
+    if spec.gate:
+        out["w_g"] = a(t["g"])
+    if spec.bias:
+        out["b_qkv"] = a(torch.cat([t["q.b"], t["k.b"], t["v.b"]], 0))
     if spec.v_mix and not spec.v_mix_first:
         out["vmix"] = f(t["vmix"]).reshape(1)
     return out
+
+
+def pack_mamba2(spec: Mamba2Spec, t: dict, device, act_dtype) -> dict:
+    """t: in ([z | x | B | C | dt] rows), conv, conv.b, dt_bias, A_log, D, norm, o.  The dt rows leave the big
+    projection for a few-row float32-output projection whose bias is dt_bias."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
+    n = 2 * spec.inner + 2 * spec.groups * spec.state
+    return dict(w_in=a(t["in"][:n]), w_dt=a(t["in"][n:]), b_dt=f(t["dt_bias"]), taps=f(t["conv"]), b_conv=f(t["conv.b"]),
+                a_log=f(t["A_log"]), skip=f(t["D"]), norm=f(t["norm"]), w_o=a(t["o"]))
+
+
+def pack_rglru(spec: RGLRUSpec, t: dict, device, act_dtype) -> dict:
+    """t: y, y.b, x, x.b, conv, conv.b, ra, ra.b, ri, ri.b, lam, o.  y | x are one biased projection; the two gate
+    matrices of a block become one float32 [blocks, in, 2 out] operand; softplus(lam) is formed once, in float32."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
+    wg = torch.cat([t["ra"].float().transpose(1, 2), t["ri"].float().transpose(1, 2)], 2)
+    bg = torch.cat([t["ra.b"].float(), t["ri.b"].float()], 1)[:, None, :]
+    return dict(w_yx=a(torch.cat([t["y"], t["x"]], 0)), b_yx=a(torch.cat([t["y.b"], t["x.b"]], 0)), taps=f(t["conv"]),
+                b_conv=f(t["conv.b"]), w_gates=f(wg), b_gates=f(bg),
+                sp=f(torch.nn.functional.softplus(t["lam"].float(), threshold=30.0)), w_o=a(t["o"]))
 
 
 def pack_delta_rule(spec: DeltaRuleSpec, t: dict, device, act_dtype) -> dict:
@@ -375,6 +501,17 @@ def pack_moe_glu(spec: MoEGluSpec, t: dict, device, act_dtype) -> dict:
         # prompt portions take the grouped matrix-core path, which wants gate and up rows interleaved per tile
         out["w_gu"] = out["w_gu"][:, hops.moe_glu_row_order(spec.ff).to(out["w_gu"].device)].contiguous()
         out["gu_tiled"] = True
+    return out
+
+
+def pack_moe_group_glu(spec: MoEGroupGluSpec, t: dict, device, act_dtype) -> dict:
+    """t: router, e<k>.gate / .up / .down and, with a shared expert, shared.gate / .up / .down / .sg."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    out = pack_moe_glu(spec, {**t, "router.b": torch.zeros(spec.experts)}, device, act_dtype)
+    del out["b_router"]
+    if spec.shared_ff:
+        out.update(ws_gu=a(torch.cat([t["shared.gate"], t["shared.up"]], 0)), ws_down=a(t["shared.down"]),
+                   ws_gate=a(t["shared.sg"].reshape(1, -1)))
     return out
 
 
@@ -449,16 +586,44 @@ def mix_latent_attention(model, li: int, spec: LatentAttentionSpec, w: dict, h, 
 
 def mix_window_attention(model, li: int, spec: WindowAttentionSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
     H, G, D, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
-    qkv = hops.matmul(h, w["w_qkv"])
-    gate = hops.rowdot(h, w["w_g"])
+    qkv = hops.matmul(h, w["w_qkv"], w.get("b_qkv"))
+    gate = hops.rowdot(h, w["w_g"]) if spec.gate else None
     mixes = spec.v_mix and not spec.v_mix_first
     v = hops.window_prep(qkv, H, G, D, Dv, meta.shared["v_first"] if mixes else None, w.get("vmix"), meta.pos,
-                         meta.tok_seq, meta.block_table, w["q_norm"], w["k_norm"], model.cfg.norm_eps,
+                         meta.tok_seq, meta.block_table, w.get("q_norm"), w.get("k_norm"), model.cfg.norm_eps,
                          model.rope.get(li), spec.rope_dims, cache.kc[li], cache.vc[li], spec.v_mix_first)
     if spec.v_mix_first:
         meta.shared["v_first"] = v
-    o = hops.window_attention(qkv, cache.kc[li], cache.vc[li], meta.block_table, meta.q_start, meta.pos, w["sink"],
-                              gate, spec.scale, spec.window, spec.keep_first, H, model.act_dtype, meta.max_q)
+    o = hops.window_attention(qkv, cache.kc[li], cache.vc[li], meta.block_table, meta.q_start, meta.pos, w.get("sink"),
+                              gate, spec.scale, spec.window, spec.keep_first, H, model.act_dtype, meta.max_q,
+                              spec.chunk)
+    return hops.matmul(o, w["w_o"])
+
+
+def mix_mamba2(model, li: int, spec: Mamba2Spec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    H, P, N, G = spec.heads, spec.vdim, spec.state, spec.groups
+    inner, GN = spec.inner, spec.groups * spec.state
+    proj = hops.matmul(h, w["w_in"])                 # z | x | B | C
+    dt_pre = hops.rowdot(h, w["w_dt"], w["b_dt"])    # float32 step pre-activations, bias included
+    xbc = hops.short_conv(proj, w["taps"], meta.tok_seq, meta.q_start, meta.pos0, meta.slots, cache.hist[li], True,
+                          w["b_conv"], inner)        # x | B | C after convolution and SiLU
+    decay, dt = hops.ssm_prep(dt_pre, w["a_log"])
+    # state rows = B, read by C, written with dt x: S <- decay S + B (dt x)^T, o = S^T C
+    o = hops.linear_scan(xbc, inner + GN, inner, 0, None, None, 1.0, decay, None, meta.q_start, meta.pos0, meta.slots,
+                         cache.S[li], G, H, N, P, dt)
+    y = hops.gated_group_norm(o, xbc, 0, w["skip"], proj, 0, w["norm"], spec.norm_groups, model.cfg.norm_eps,
+                              model.act_dtype)
+    return hops.matmul(y, w["w_o"])
+
+
+def mix_rglru(model, li: int, spec: RGLRUSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    W = spec.width
+    proj = hops.matmul(h, w["w_yx"], w["b_yx"])      # y branch | x branch
+    u = hops.short_conv(proj, w["taps"], meta.tok_seq, meta.q_start, meta.pos0, meta.slots, cache.hist[li], False,
+                        w["b_conv"], W)
+    gates = hops.block_gates(u, w["w_gates"], w["b_gates"])   # float32 [blocks, T, 2 W / blocks]
+    o = hops.rglru_scan(u, gates, w["sp"], spec.c, proj, 0, meta.q_start, meta.pos0, meta.slots, cache.S[li],
+                        model.act_dtype, meta.max_q)
     return hops.matmul(o, w["w_o"])
 
 
@@ -496,6 +661,19 @@ def ff_moe_glu(model, spec: MoEGluSpec, w: dict, h):
                             bool(w.get("gu_tiled", False)))
 
 
+def ff_moe_group_glu(model, spec: MoEGroupGluSpec, w: dict, h):
+    """Returns the routed experts' sum and, with a shared expert, (sum, shared output, float32 gate logits [T, 1]):
+    the stream's join adds sigmoid(gate) * shared."""
+    idx, wt = hops.moe_route_group(h, w["w_router"], spec.top, spec.groups, spec.keep, spec.scale)
+    y = hops.moe_glu_ffn(h, idx, wt, w["w_gu"], w["w_down"], spec.limit, spec.slope, spec.shift, model.act_dtype,
+                         bool(w.get("gu_tiled", False)))
+    if not spec.shared_ff:
+        return y
+    ys = hops.matmul(hops.glu(hops.matmul(h, w["ws_gu"]), spec.limit, spec.slope, spec.shift, model.act_dtype),
+                     w["ws_down"])
+    return y, ys, hops.rowdot(h, w["ws_gate"])
+
+
 def ff_dense(model, spec: DenseFFSpec, w: dict, h):
     return hops.matmul(hops.act_inplace(hops.matmul(h, w["w_up"]), spec.act), w["w_down"])
 
@@ -507,10 +685,11 @@ def ff_moe(model, spec: MoEFFSpec, w: dict, h):
 
 MIXERS = {"mlstm": (mix_mlstm, pack_mlstm), "latent_attention": (mix_latent_attention, pack_latent),
           "window_attention": (mix_window_attention, pack_window_attention),
-          "delta_rule": (mix_delta_rule, pack_delta_rule), "gla": (mix_gla, pack_gla)}
+          "delta_rule": (mix_delta_rule, pack_delta_rule), "gla": (mix_gla, pack_gla),
+          "mamba2": (mix_mamba2, pack_mamba2), "rglru": (mix_rglru, pack_rglru)}
 FEED_FORWARDS = {"dense": (ff_dense, pack_dense), "moe": (ff_moe, pack_moe), "glu": (ff_glu, pack_glu),
-                 "moe_glu": (ff_moe_glu, pack_moe_glu)}
-RECURRENT_MIXERS = ("mlstm", "delta_rule", "gla")
+                 "moe_glu": (ff_moe_glu, pack_moe_glu), "moe_group_glu": (ff_moe_group_glu, pack_moe_group_glu)}
+RECURRENT_MIXERS = ("mlstm", "delta_rule", "gla", "mamba2", "rglru")
 
 
 # -----------------------------------------------------------------------------------------------------------------
@@ -537,13 +716,15 @@ class HybridDecoder:
         self.sequence_parallel = False
         self.decode_overlap_rows = 0
         P = max_position or cfg.max_position
-        self.rope = {li: rope_cos_sin(l.mixer.rope_base, l.mixer.rope_dims, P, self.device,
+        self.rope = {ri: rope_cos_sin(l.mixer.rope_base, l.mixer.rope_dims, P, self.device,
                                       getattr(l.mixer, "rope_scaling", None))
-                     for li, l in enumerate(cfg.layers)
+                     for ri, l in enumerate(cfg.layers[i] for i in cfg.runs)
                      if l.mixer.kind in ("latent_attention", "window_attention") and l.mixer.rope_dims}
         self.recurrent = any(l.mixer.kind in RECURRENT_MIXERS for l in cfg.layers)
-        if cfg.residual not in ("out_norm", "post_norm"):
+        if cfg.residual not in ("out_norm", "post_norm", "pre_norm"):
             raise ValueError(f"unknown residual rule {cfg.residual!r}")
+        if cfg.token_side and cfg.residual != "pre_norm":
+            raise ValueError("the per-layer token input is part of the pre-norm stream's join")
 
     # ---- what the engine calls --------------------------------------------------------------------------------
     def make_cache(self, num_blocks: int, block_size: int, slots: int, kv_dtype: str = "bf16", k_scale: float = 1.0,
@@ -604,25 +785,60 @@ class HybridDecoder:
         cfg, w, at = self.cfg, self.w, self.act_dtype
         meta = self._meta(sb)
         x, h = hops.embed_rows(meta.ids, w.embed, at)
-        for li, (spec, lw) in enumerate(zip(cfg.layers, w.layers)):
-            y = MIXERS[spec.mixer.kind][0](self, li, spec.mixer, lw.mix, h, meta, cache)
-            h = self._join(y, x, lw.norm1)
-            if spec.ff is not None:
-                y = FEED_FORWARDS[spec.ff.kind][0](self, spec.ff, lw.ff, h)
-                h = self._join(y, x, lw.norm2)
-            if self.layer_tap is not None:
-                self.layer_tap(li, x)
+        if cfg.residual == "pre_norm":
+            self._forward_pre_norm(x, meta, cache)
+        else:
+            for ri, li in enumerate(cfg.runs):   # the cache is keyed by run, the weights by layer
+                spec, lw = cfg.layers[li], w.layers[li]
+                y = MIXERS[spec.mixer.kind][0](self, ri, spec.mixer, lw.mix, h, meta, cache)
+                h = self._join(y, x, lw.norm1)
+                if spec.ff is not None:
+                    y = FEED_FORWARDS[spec.ff.kind][0](self, spec.ff, lw.ff, h)
+                    h = self._join(y, x, lw.norm2)
+                if self.layer_tap is not None:
+                    self.layer_tap(ri, x)
         xs = x.index_select(0, meta.last_idx)
-        final = hops.rms_norm if cfg.residual == "post_norm" else hops.layer_norm
+        final = hops.layer_norm if cfg.residual == "out_norm" else hops.rms_norm
         logits = hops.matmul(final(xs, w.final_norm, cfg.norm_eps, at), w.head).float()
         if cfg.logit_scale != 1.0:
             logits = logits * cfg.logit_scale
         return logits if logits.dtype == logits_dtype else logits.to(logits_dtype)
 
+    def _forward_pre_norm(self, x, meta: StepMeta, cache: HybridCache) -> None:
+        """x <- x + mixer(norm1(x)); x <- x + ff(norm2(x)); with a per-layer token input
+        x <- x + rms_unit(W_proj (gelu(W_gate x) * e)) * w, e the layer's columns of each token's row of a second
+        embedding table.  Every join kernel adds to the float32 stream in place and emits what the next sublayer
+        reads: the next norm's output, or the stream's copy in the activation dtype for the token input's gate."""
+        cfg, w, at, eps = self.cfg, self.w, self.act_dtype, self.cfg.norm_eps
+        runs = cfg.runs
+        h = hops.rms_norm(x, w.layers[runs[0]].norm1, eps, at) if runs else None
+        for ri, li in enumerate(runs):
+            spec, lw = cfg.layers[li], w.layers[li]
+            nxt = w.layers[runs[ri + 1]].norm1 if ri + 1 < len(runs) else None   # the last run emits nothing:
+            last = ri + 1 == len(runs)                                           # the final norm reads chosen rows
+            y = MIXERS[spec.mixer.kind][0](self, ri, spec.mixer, lw.mix, h, meta, cache)
+            y2 = g2 = None
+            if spec.ff is not None:
+                h = hops.add_rms_norm(y, x, lw.norm2, eps, at)
+                y = FEED_FORWARDS[spec.ff.kind][0](self, spec.ff, lw.ff, h)
+                if isinstance(y, tuple):
+                    y, y2, g2 = y
+            if cfg.token_side:
+                xa = hops.add_rms_norm(y, x, None, eps, at, y2, g2)
+                g = hops.token_gate(hops.matmul(xa, lw.side["w_gate"]), meta.ids, w.side_embed, lw.side["col0"], at)
+                h = hops.add_rms_norm(hops.matmul(g, lw.side["w_proj"]), x, nxt, eps, at, w_y=lw.side["norm"],
+                                      emit=not last)
+            else:
+                h = hops.add_rms_norm(y, x, nxt, eps, at, y2, g2, emit=not last)
+            if self.layer_tap is not None:
+                self.layer_tap(ri, x)
+
     def _join(self, y, x, w):
         """The residual rule: folds the sublayer output y into the float32 stream x (in place) and returns the
         stream in the activation dtype for the next sublayer."""
         cfg = self.cfg
+        if isinstance(y, tuple):
+            raise NotImplementedError("a feed-forward with a separately gated part needs the pre-norm stream")
         if cfg.residual == "post_norm":
             return hops.scale_add_rms_norm(y, x, w, cfg.residual_alpha, cfg.norm_eps, self.act_dtype)
         return hops.add_layer_norm(y, x, w, cfg.norm_eps, self.act_dtype)

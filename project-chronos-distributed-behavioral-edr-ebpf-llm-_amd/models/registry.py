@@ -147,6 +147,29 @@ def _kalesun_presets():
     return list(kalesun.PRESETS)
 
 
+def _tugovik_build(name, device, tp, seed, is_path, max_position, weight_dtype, dtype):
+    from . import tugovik
+
+    if tp.world > 1:
+        raise NotImplementedError("Tugovik runs on full-weight ranks (data-parallel replicas)")
+    if weight_dtype != "bf16":
+        raise NotImplementedError("Tugovik weights are served in the activation dtype (no fp8 projections)")
+    return tugovik.build(name, device, seed, DTYPES[dtype], max_position)
+
+
+def _tugovik_is_checkpoint(path: str) -> bool:
+    from . import tugovik
+
+    return tugovik.is_checkpoint(path)
+
+
+def _tugovik_presets():
+    from . import tugovik
+
+    return list(tugovik.PRESETS)
+
+
+register(Family("tugovik", _tugovik_presets, _tugovik_is_checkpoint, _tugovik_build, ("bf16", "fp32")))
 register(Family("kalesun", _kalesun_presets, _kalesun_is_checkpoint, _kalesun_build, ("bf16", "fp32")))
 register(Family("zokunex", _zokunex_presets, _zokunex_is_checkpoint, _zokunex_build, ("bf16", "fp32")))
 register(Family("llama", _llama_presets, _llama_is_checkpoint, _llama_build, ("bf16",)))

@@ -47,8 +47,12 @@ def _f32(act_dtype) -> bool:
     return act_dtype == torch.float32
 
 
-def matmul(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
-    """x @ w.T: the framework's routed projection GEMMs for bfloat16, the library's float32 GEMM otherwise."""
+def matmul(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+    """x @ w.T (+ bias): the framework's routed projection GEMMs for bfloat16, the library's float32 GEMM otherwise.
+    A biased projection is one library GEMM whose epilogue adds the bias (in the activation dtype, like w) to the
+    float accumulator before the rounding."""
+    if bias is not None:
+        return torch.addmm(bias, x, w.t())
     if x.dtype == torch.bfloat16:
         from . import linear
 
@@ -166,19 +170,20 @@ def window_prep(qkv, H: int, G: int, D: int, Dv: int, v_first, lam, pos, tok_seq
 
 
 def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale: float, window: int, keep_first: int,
-                     H: int, act_dtype, max_q: int):
-    """``max_q``: the most tokens any sequence brings in this step (sizes the launch grid)."""
+                     H: int, act_dtype, max_q: int, chunk: int = 0):
+    """``max_q``: the most tokens any sequence brings in this step (sizes the launch grid).  ``chunk`` > 0: keys
+    outside the query's own chunk of that many positions are hidden."""
     if _gpu(qkv):
         return _k().hy_window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first,
-                                        H, max_q)
+                                        chunk, H, max_q)
     return ref.window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H,
-                                act_dtype)
+                                act_dtype, chunk)
 
 
-def short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu: bool = True):
+def short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu: bool = True, bias=None, x_off: int = 0):
     if _gpu(x):
-        return _k().hy_short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu)
-    return ref.short_conv(x, w, q_start, pos0, slots, hist, silu)
+        return _k().hy_short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu, bias, x_off)
+    return ref.short_conv(x, w, q_start, pos0, slots, hist, silu, bias, x_off)
 
 
 def delta_prep(y, ab, a_log, HK: int, H: int, D: int, q_mul: float):
@@ -195,12 +200,12 @@ def decay_pow(z, inv_tau: float):
 
 
 def linear_scan(proj, q_off: int, k_off: int, v_off: int, qscale, kscale, q_mul: float, decay, beta, q_start, pos0,
-                slots, S, HK: int, H: int, D: int, Dv: int):
+                slots, S, HK: int, H: int, D: int, Dv: int, vscale=None):
     if _gpu(proj):
         return _k().hy_linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots,
-                                   S, HK, H, D, Dv)
+                                   S, HK, H, D, Dv, vscale)
     return ref.linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots, S, HK,
-                           H, D, Dv)
+                           H, D, Dv, vscale)
 
 
 def head_norm_gate(o, src, g_off: int, w, eps: float, silu_gate: bool, act_dtype):
@@ -234,3 +239,58 @@ def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit: float, slope: float, shift: flo
     if tiled:
         w_gu = w_gu[:, torch.argsort(moe_glu_row_order(w_gu.shape[1] // 2)).to(w_gu.device)]
     return ref.moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift, act_dtype)
+
+
+# ---- pre-norm residual stream, per-layer token input, state-space and gated linear recurrences, grouped router ---
+
+
+def add_rms_norm(y, x, w_out, eps: float, act_dtype, y2=None, gate2=None, w_y=None, emit: bool = True):
+    """x (float32 residual, in place) <- x + v, v = y (+ sigmoid(gate2) y2), divided by its own root mean square and
+    times w_y when that is given.  Returns in the activation dtype rms_norm(x) * w_out, or the updated rows
+    themselves when w_out is None (x itself for float32), or None when ``emit`` is off."""
+    if _gpu(x):
+        h = _k().hy_add_rms_norm(y, x, w_out, eps, _f32(act_dtype), y2, gate2, w_y, emit)
+        if not emit:
+            return None
+        return x if (w_out is None and _f32(act_dtype)) else h
+    return ref.add_rms_norm(y, x, w_out, eps, act_dtype, y2, gate2, w_y, emit)
+
+
+def token_gate(a, ids, table, col0: int, act_dtype):
+    if _gpu(a):
+        return _k().hy_token_gate(a, ids, table, col0)
+    return ref.token_gate(a, ids, table, col0, act_dtype)
+
+
+def ssm_prep(dt_pre, a_log):
+    if _gpu(dt_pre):
+        return _k().hy_ssm_prep(dt_pre, a_log)
+    return ref.ssm_prep(dt_pre, a_log)
+
+
+def gated_group_norm(o, skip_src, skip_off: int, skip_w, gate_src, g_off: int, w, groups: int, eps: float, act_dtype):
+    if _gpu(o):
+        return _k().hy_gated_group_norm(o, skip_src, skip_off, skip_w, gate_src, g_off, w, groups, eps, _f32(act_dtype))
+    return ref.gated_group_norm(o, skip_src, skip_off, skip_w, gate_src, g_off, w, groups, eps, act_dtype)
+
+
+def block_gates(u, w_gates, b_gates):
+    """Gate pre-activations of a block-diagonal projection, float32: u [T, W] split into NB blocks of channels, block b
+    times w_gates[b] ([W / NB, n]) plus b_gates[b] ([1, n]).  Returns [NB, T, n].  A float32 library product on both
+    devices and in both activation dtypes (its outputs are gates of a recurrence)."""
+    NB = w_gates.shape[0]
+    T, W = u.shape
+    return torch.baddbmm(b_gates, u.float().view(T, NB, W // NB).transpose(0, 1), w_gates)
+
+
+def rglru_scan(u, gates, sp, c: float, ysrc, y_off: int, q_start, pos0, slots, S, act_dtype, max_q: int = 0):
+    """``max_q``: the most tokens any sequence brings in this step (sizes the launch grid; 0 = unknown)."""
+    if _gpu(u):
+        return _k().hy_rglru_scan(u, gates.contiguous(), sp, c, ysrc, y_off, q_start, pos0, slots, S, max_q)
+    return ref.rglru_scan(u, gates, sp, c, ysrc, y_off, q_start, pos0, slots, S, act_dtype)
+
+
+def moe_route_group(h, w_router, top: int, n_groups: int, keep: int, scale: float):
+    if _gpu(h):
+        return _k().hy_moe_route_group(h, w_router, top, n_groups, keep, scale)
+    return ref.moe_route_group(h, w_router, top, n_groups, keep, scale)

@@ -214,8 +214,8 @@ def glu(gu, limit, slope, shift, act_dtype):
 
 def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin, dims, kc, vc,
                 emit_v):
-    """qkv [T, H D + G D + G Dv]: per-head RMS norm (weights q_norm / k_norm [D], float32 math) and rotation of the
-    query and key heads, queries in place; values mixed with ``v_first`` [T, G Dv] as (1 - lam) v + lam v_first when
+    """qkv [T, H D + G D + G Dv]: per-head RMS norm (weights q_norm / k_norm [D], float32 math; both None: no
+    norm) and rotation of the query and key heads, queries in place; values mixed with ``v_first`` [T, G Dv] as (1 - lam) v + lam v_first when
     given; keys and (mixed) values written to the paged caches kc [NB, BS, G, D], vc [NB, BS, G, Dv].  Returns the
     values as read from the projection [T, G Dv] when ``emit_v`` (the source of later layers' mixing), else None."""
     T = qkv.shape[0]
@@ -226,7 +226,8 @@ def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_nor
 
     def norm_rot(x, w):
         xf = x.float()
-        xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
+        if w is not None:
+            xf = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()
         return rotate_half_rows(xf, cos_sin, pos, dims) if dims else xf
 
     qn = norm_rot(q, q_norm)
@@ -243,9 +244,12 @@ def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_nor
     return out_v
 
 
-def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H, act_dtype):
+def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H, act_dtype,
+                     chunk=0):
     """Causal softmax attention over a paged cache through a sliding window that also keeps a sequence's first
     tokens: the query at position i sees key j <= i when i - j < window or j < keep_first (window 0: every j <= i).
+    ``chunk`` > 0 further hides every key outside the query's own chunk of that many positions, counted from
+    position 0 of the sequence: j is visible only when j // chunk == i // chunk.
     ``sink`` f32 [H] or None: exp(sink_h) joins the softmax denominator (no key, no value).  ``gate`` f32 [T, H] or
     None: head h's output times sigmoid(gate).  Queries are the first H D columns of qkv; query head h reads
     key/value head h // (H / G).  Returns [T, H Dv]."""
@@ -271,6 +275,8 @@ def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, 
         hidden = j > p[:, None]
         if window:
             hidden = hidden | ((p[:, None] - j >= window) & (j >= keep_first))
+        if chunk:
+            hidden = hidden | (j < (p[:, None] // chunk) * chunk)
         sc = sc.masked_fill(hidden[:, None, :], float("-inf"))
         if sink is not None:
             sc = torch.cat([sc, sink.float()[None, :, None].expand(t1 - t0, H, 1)], -1)
@@ -281,13 +287,13 @@ def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, 
     return out.reshape(T, H * Dv).to(act_dtype)
 
 
-def short_conv(x, w, q_start, pos0, slots, hist, silu):
-    """Causal per-channel convolution over time on a flattened token stream, on the first C columns of x [T, >= C];
-    w f32 [C, K] (the last column weighs the current token); hist [NS, K - 1, C]: every sequence's last K - 1 inputs
-    (oldest first), read when its range starts past position 0 (zeros otherwise) and updated in place.  Returns
-    [T, C] in x's dtype."""
+def short_conv(x, w, q_start, pos0, slots, hist, silu, bias=None, x_off=0):
+    """Causal per-channel convolution over time on a flattened token stream, on the C columns of x [T, >= x_off + C]
+    from column x_off on; w f32 [C, K] (the last column weighs the current token), bias f32 [C] or None; hist
+    [NS, K - 1, C]: every sequence's last K - 1 inputs (oldest first), read when its range starts past position 0
+    (zeros otherwise) and updated in place.  Returns [T, C] in x's dtype."""
     C, K = w.shape
-    x = x[:, :C]
+    x = x[:, x_off:x_off + C]
     y = torch.empty_like(x)
     qs, p0, sl = q_start.tolist(), pos0.tolist(), slots.tolist()
     for b in range(len(sl)):
@@ -299,6 +305,8 @@ def short_conv(x, w, q_start, pos0, slots, hist, silu):
         acc = torch.zeros(t1 - t0, C, dtype=torch.float32, device=x.device)
         for i in range(K):
             acc += ext[i:i + t1 - t0] * w[:, i].float()
+        if bias is not None:
+            acc += bias.float()
         if silu:
             acc = acc * torch.sigmoid(acc)
         y[t0:t1] = acc.to(x.dtype)
@@ -327,7 +335,8 @@ def decay_pow(z, inv_tau):
     return z
 
 
-def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots, S, HK, H, D, Dv):
+def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, pos0, slots, S, HK, H, D, Dv,
+                vscale=None):
     """Linear-state recurrence over a flattened token stream, per value head h (reading q/k head h // (H / HK)):
 
         S <- decay * S                      decay f32 [T, H] (one per head) or [T, H, D] (one per key channel / row)
@@ -335,8 +344,9 @@ def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q
         S <- S + k u^T;   o = S^T q
 
     q, k, v are columns of proj [T, C] at q_off / k_off / v_off; q is multiplied by qscale [T, HK] (or by q_mul when
-    None) and k by kscale [T, HK] (when given), in float32.  S f32 [NS, H, D, Dv] by slot, in place; a range whose
-    first token sits at position 0 starts from zero.  Returns o f32 [T, H, Dv]."""
+    None), k by kscale [T, HK] (when given) and v by vscale [T, H] (when given; not with beta), in float32.  S f32
+    [NS, H, D, Dv] by slot, in place; a range whose first token sits at position 0 starts from zero.  Returns o f32
+    [T, H, Dv]."""
     T = proj.shape[0]
     out = torch.zeros(T, H, Dv, dtype=torch.float32, device=proj.device)
     qs, p0, sl = q_start.tolist(), pos0.tolist(), slots.tolist()
@@ -347,6 +357,8 @@ def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q
     q = q * (qscale[:, :, None] if qscale is not None else q_mul)
     if kscale is not None:
         k = k * kscale[:, :, None]
+    if vscale is not None:
+        v = v * vscale[:, :, None]
     rep = H // HK
     q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
     dec = decay.view(T, H, -1, 1)  # [T, H, 1 | D, 1]
@@ -398,3 +410,103 @@ def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit, slope, shift, act_dtype):
         y = (glu(gu, limit, slope, shift, act_dtype) @ w_down[e].t().to(act_dtype)).float()
         out.index_add_(0, tok, y * wt[tok, kk][:, None])
     return out.to(act_dtype)
+
+
+# ---- pre-norm residual stream, per-layer token input, state-space and gated linear recurrences, grouped router ---
+
+
+def gelu_tanh(z):
+    return 0.5 * z * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (z + 0.044715 * z * z * z)))
+
+
+def add_rms_norm(y, x, w_out, eps, act_dtype, y2=None, gate2=None, w_y=None, emit=True):
+    """The pre-norm stream's join.  v = y (+ sigmoid(gate2) * y2, gate2 f32 [T, 1]); when w_y is given v is first
+    divided by its own root mean square and multiplied by w_y; x (float32, in place) <- x + v.  Returns, in the
+    activation dtype, rms_norm(x) * w_out when w_out is given, else x itself (None when ``emit`` is off)."""
+    v = y.float()
+    if y2 is not None:
+        v = v + torch.sigmoid(gate2.float().reshape(-1, 1)) * y2.float()
+    if w_y is not None:
+        v = v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + eps) * w_y.float()
+    x.add_(v)
+    if not emit:
+        return None
+    if w_out is None:
+        return x if act_dtype == torch.float32 else x.to(act_dtype)
+    return rms_norm(x, w_out, eps, act_dtype)
+
+
+def token_gate(a, ids, table, col0, act_dtype):
+    """gelu_tanh(a) * table[ids, col0 : col0 + a.shape[1]]: a projection gated by each token's own row of a table."""
+    e = table[ids.long(), col0:col0 + a.shape[1]].float()
+    return (gelu_tanh(a.float()) * e).to(act_dtype)
+
+
+def ssm_prep(dt_pre, a_log):
+    """Per token and head of a state-space layer: step dt = softplus(dt_pre) (bias already added, no clamp) and
+    decay = exp(-exp(a_log) dt).  dt_pre f32 [T, H].  Returns float32 (decay, dt)."""
+    dt = torch.nn.functional.softplus(dt_pre.float(), threshold=30.0)
+    return torch.exp(-torch.exp(a_log.float()) * dt), dt
+
+
+def gated_group_norm(o, skip_src, skip_off, skip_w, gate_src, g_off, w, groups, eps, act_dtype):
+    """Read-out of a state-space layer: y = (o + skip_w[h] * x) * silu(z) with x = skip_src[:, skip_off:...] and
+    z = gate_src[:, g_off:...] (both [T, H Dv] column ranges), then RMS norm in ``groups`` equal parts of the H Dv
+    columns (each part by its own root mean square), times w [H Dv].  o f32 [T, H, Dv]."""
+    T, H, Dv = o.shape
+    n = H * Dv
+    y = o + skip_w.float()[None, :, None] * skip_src[:, skip_off:skip_off + n].float().view(T, H, Dv)
+    z = gate_src[:, g_off:g_off + n].float()
+    y = y.reshape(T, n) * (z * torch.sigmoid(z))
+    y = y.view(T, groups, n // groups)
+    y = y * torch.rsqrt(y.pow(2).mean(-1, keepdim=True) + eps)
+    return (y.reshape(T, n) * w.float()).to(act_dtype)
+
+
+def rglru_scan(u, gates, sp, c, ysrc, y_off, q_start, pos0, slots, S, act_dtype):
+    """Real-gated linear recurrent unit over a flattened token stream, per channel:
+
+        r = sigmoid(gates[.., 0, :]),  i = sigmoid(gates[.., 1, :]),  log a = -c r sp,  a = exp(log a)
+        S <- a S + sqrt(1 - a^2) i u;     out = S * gelu_tanh(y)
+
+    u [T, W] (the convolved branch); gates f32 [NB, T, 2 W / NB]: per block of channels the pre-activations of r, then of i;
+    sp f32 [W] = softplus of the decay parameter; y = ysrc[:, y_off : y_off + W]; S f32 [NS, W] by slot, in place; a
+    range whose first token sits at position 0 starts from zero.  Returns [T, W] in the activation dtype."""
+    T, W = u.shape
+    NB = gates.shape[0]
+    g = gates.float().reshape(NB, T, 2, W // NB).permute(1, 2, 0, 3).reshape(T, 2, W)
+    r, i = torch.sigmoid(g[:, 0]), torch.sigmoid(g[:, 1])
+    log_a = -c * r * sp.float()
+    a = torch.exp(log_a)
+    b = torch.sqrt(-torch.expm1(2.0 * log_a)) * i * u.float()
+    out = torch.empty(T, W, dtype=torch.float32, device=u.device)
+    qs, p0, sl = q_start.tolist(), pos0.tolist(), slots.tolist()
+    for bb in range(len(sl)):
+        if qs[bb + 1] <= qs[bb]:
+            continue
+        s = torch.zeros_like(S[sl[bb]]) if p0[bb] == 0 else S[sl[bb]].clone()
+        for t in range(qs[bb], qs[bb + 1]):
+            s = a[t] * s + b[t]
+            out[t] = s
+        S[sl[bb]] = s
+    return (out * gelu_tanh(ysrc[:, y_off:y_off + W].float())).to(act_dtype)
+
+
+def moe_route_group(h, w_router, top, n_groups, keep, scale):
+    """Router with sigmoid scores and a choice limited to the best groups: the N outputs form n_groups equal groups
+    of neighbours, a group scores the sum of its two largest scores, the ``keep`` best groups stay, and the ``top``
+    largest scores among them are chosen (ties: the lower index) and weighted by score / (sum of the chosen + 1e-20)
+    * scale.  Returns (idx int32 [T, top], weight f32 [T, top])."""
+    s = torch.sigmoid(rowdot(h, w_router))
+    T, N = s.shape
+    cand = s
+    if n_groups > 1 and keep < n_groups:
+        per = N // n_groups
+        gs = s.view(T, n_groups, per).topk(min(2, per), dim=-1).values.sum(-1)
+        # stable choice of the best groups: by score, then by the lower index
+        order = torch.sort(gs, dim=-1, descending=True, stable=True).indices[:, :keep]
+        ok = torch.zeros(T, n_groups, dtype=torch.bool, device=s.device).scatter_(1, order, True)
+        cand = s.masked_fill(~ok[:, :, None].expand(T, n_groups, per).reshape(T, N), float("-inf"))
+    idx = torch.sort(cand, dim=-1, descending=True, stable=True).indices[:, :top]
+    val = torch.gather(s, 1, idx)
+    return idx.to(torch.int32), val / (val.sum(-1, keepdim=True) + 1e-20) * scale
