@@ -46,7 +46,7 @@ def chunk_visible(i, j, size):
 def attention_token(h, W, p, mx, pos, cache):
     """One token of the chunked attention mixer.  cache: list of (k [G, D], v [G, Dv]) of ALL earlier tokens; this
     token's pair is appended."""
-    H, G, D, Dv = mx["heads"], mx["kv_heads"], mx["dim"], mx["vdim"]
+    H, G, D, Dv = mx["heads"], mx.get("kv_heads", mx["heads"]), mx["dim"], mx["vdim"]
     q = (W[p + "q"] @ h + W[p + "q.b"]).view(H, D)
     k = (W[p + "k"] @ h + W[p + "k.b"]).view(G, D)
     v = (W[p + "v"] @ h + W[p + "v.b"]).view(G, Dv)
@@ -79,7 +79,7 @@ def conv_token(u, taps, bias, hist):
 
 def mamba2_token(h, W, p, mx, eps, state):
     """One token of the state-space mixer.  state: dict with 'S' [heads, N, P] and 'hist' (list of conv inputs)."""
-    Hn, P, N, G = mx["heads"], mx["vdim"], mx["state"], mx["groups"]
+    Hn, P, N, G = mx["heads"], mx["vdim"], mx["state"], mx.get("groups", 1)
     inner = Hn * P
     zx = W[p + "in"] @ h
     z, xbc, dt = zx[:inner], zx[inner:2 * inner + 2 * G * N], zx[2 * inner + 2 * G * N:]
@@ -95,14 +95,14 @@ def mamba2_token(h, W, p, mx, eps, state):
         state["S"][hd] = decay * state["S"][hd] + dt[hd] * torch.outer(Bm[g], x[hd])
         y[hd] = state["S"][hd].t() @ Cm[g] + W[p + "D"][hd] * x[hd]
     y = y.reshape(-1) * silu(z)
-    ng = mx["norm_groups"]
+    ng = mx.get("norm_groups", 1)
     y = rms_unit(y.view(ng, inner // ng), eps).reshape(-1) * W[p + "norm"]
     return W[p + "o"] @ y
 
 
 def rglru_token(h, W, p, mx, state):
     """One token of the gated linear recurrent mixer.  state: dict with 'S' [width] and 'hist'."""
-    Wd, nb = mx["width"], mx["blocks"]
+    Wd, nb = mx["width"], mx.get("blocks", 1)
     y = gelu_tanh(W[p + "y"] @ h + W[p + "y.b"])
     u = conv_token(W[p + "x"] @ h + W[p + "x.b"], W[p + "conv"], W[p + "conv.b"], state["hist"])
     ub = u.view(nb, Wd // nb)
@@ -126,7 +126,7 @@ def route(h, W, p, r):
     allowed = torch.ones(E, dtype=torch.bool)
     grp = r.get("groups")
     if grp:
-        n, keep = grp["count"], grp["keep"]
+        n, keep = grp["count"], grp.get("keep", grp["count"])
         per = E // n
         gs = [float(torch.sort(s[g * per:(g + 1) * per], descending=True).values[:2].sum()) for g in range(n)]
         best = sorted(range(n), key=lambda g: (-gs[g], g))[:keep]
@@ -180,7 +180,7 @@ class PlainTugovik:
             if l["type"] == "attention":
                 self.state.append([])
             elif l["type"] == "mamba2":
-                ch = mx["heads"] * mx["vdim"] + 2 * mx["groups"] * mx["state"]
+                ch = mx["heads"] * mx["vdim"] + 2 * mx.get("groups", 1) * mx["state"]
                 self.state.append({"S": torch.zeros(mx["heads"], mx["state"], mx["vdim"], dtype=F),
                                    "hist": [torch.zeros(ch, dtype=F) for _ in range(mx["conv"] - 1)]})
             elif l["type"] == "rglru":
@@ -213,3 +213,15 @@ class PlainTugovik:
         logits = W["head"] @ offset_norm(x, W["final.norm"], eps)
         self.pos += 1
         return logits, streams
+
+
+def run(cfg: dict, tensors: dict, tokens):
+    """Logits of every token [n, vocab] and the stream after every layer run [runs][n, width]."""
+    m = PlainTugovik(cfg, tensors)
+    logits, per_run = [], [[] for _ in m.runs]
+    for t in tokens:
+        lg, streams = m.step(int(t))
+        logits.append(lg)
+        for r, x in enumerate(streams):
+            per_run[r].append(x)
+    return torch.stack(logits), [torch.stack(v) for v in per_run]

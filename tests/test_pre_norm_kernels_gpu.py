@@ -205,7 +205,7 @@ def test_chunked_attention(dt, H, G, D, Dv, chunk, window):
     from chronos.ops import hybrid as hops, hybrid_ref as ref
 
     g = _gen(H * D + chunk)
-    bs, nb = 16, 96
+    bs, nb = 16, 256
     lens, starts = [37, 1, 150, 1, 2, 1, 70], [0, 2 * chunk, 60, 0, 3 * chunk - 1, 4 * chunk - 1, 130]
     pos, seq, bt, qs = _stream(lens, starts, bs, nb)
     T = int(qs[-1])
