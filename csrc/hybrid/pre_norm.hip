@@ -35,6 +35,20 @@ template <> __device__ __forceinline__ void pn_st4<uint16_t>(uint16_t* p, const 
 __device__ __forceinline__ float gelu_tanhf_(float z) {
     return 0.5f * z * (1.f + tanhf(0.7978845608028654f * (z + 0.044715f * z * z * z)));
 }
+// The scan's per-token math on the hardware's exp2 and reciprocal (each good to about one unit in the last place):
+// a token costs a wave two sigmoids, an exponential, 1 - exp(x), a root and a tanh, and the library forms of these
+// (range reduction, IEEE division) made the scan ALU-bound.
+__device__ __forceinline__ float fast_exp_(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float fast_sigmoid_(float x) { return __builtin_amdgcn_rcpf(1.f + fast_exp_(-x)); }
+// 1 - exp(x) for x <= 0: the series near zero (where the subtraction would cancel), the exponential elsewhere
+__device__ __forceinline__ float one_minus_exp_(float x) {
+    const float p = -x * (1.f + x * (0.5f + x * (1.f / 6.f + x * (1.f / 24.f + x * (1.f / 120.f + x * (1.f / 720.f))))));
+    return x > -0.25f ? p : 1.f - fast_exp_(x);
+}
+__device__ __forceinline__ float fast_gelu_tanh_(float z) {
+    const float t = 0.7978845608028654f * (z + 0.044715f * z * z * z);   // tanh(t) = 1 - 2 / (exp(2t) + 1)
+    return 0.5f * z * (2.f - 2.f * __builtin_amdgcn_rcpf(fast_exp_(2.f * t) + 1.f));
+}
 __device__ __forceinline__ float softplusf_(float z) { return z > 30.f ? z : log1pf(expf(z)); }
 
 // emit: 0 nothing, 1 the updated row, 2 its RMS norm times w_out.  VEC: d % 4 == 0 (16-byte accesses).
@@ -222,12 +236,12 @@ __global__ void __launch_bounds__(256) rglru_scan_kernel(const T* __restrict__ u
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int t = min(tb + e, t1 - 1);
-            const float r = sigmoidf_(gr[(int64_t)t * 2 * bw]);
-            const float ig = sigmoidf_(gr[(int64_t)t * 2 * bw + bw]);
+            const float r = fast_sigmoid_(gr[(int64_t)t * 2 * bw]);
+            const float ig = fast_sigmoid_(gr[(int64_t)t * 2 * bw + bw]);
             const float la = -cc * r * spc;
-            a[e] = expf(la);
-            m[e] = sqrtf(-expm1f(2.f * la)) * ig * ld<T>(u + (int64_t)t * W + c);
-            if (PHASE == 2) g[e] = gelu_tanhf_(ld<T>(ys + (int64_t)t * ldy + y_off + c));
+            a[e] = fast_exp_(la);
+            m[e] = __builtin_amdgcn_sqrtf(one_minus_exp_(2.f * la)) * ig * ld<T>(u + (int64_t)t * W + c);
+            if (PHASE == 2) g[e] = fast_gelu_tanh_(ld<T>(ys + (int64_t)t * ldy + y_off + c));
         }
 #pragma unroll
         for (int e = 0; e < 4; ++e) {

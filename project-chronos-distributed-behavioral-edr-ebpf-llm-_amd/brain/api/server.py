@@ -220,9 +220,9 @@ def main(argv=None) -> int:
     ap.add_argument("--port", type=int, default=11434)
     ap.add_argument("--model", default="llama3-8b",
                     help="preset of any registered family (random-init) when --checkpoint is not given, e.g. llama3-8b, "
-                         "zokunex-1b, kalesun-tiny, kalesun-1b; or a checkpoint directory")
+                         "zokunex-1b, kalesun-tiny, kalesun-1b, tugovik-tiny, tugovik-1b; or a checkpoint directory")
     ap.add_argument("--checkpoint", default=None,
-                    help="checkpoint directory: HF or Meta Llama-3, or a Zokunex / Kalesun config.json + model.safetensors")
+                    help="checkpoint directory: HF or Meta Llama-3, or a Zokunex / Kalesun / Tugovik config.json + model.safetensors")
     ap.add_argument("--dtype", choices=["bf16", "fp32"], default="bf16",
                     help="activation / weight dtype (fp32: the families that run in it)")
     ap.add_argument("--tokenizer", default=None)

@@ -453,13 +453,14 @@ def pack_mamba2(spec: Mamba2Spec, t: dict, device, act_dtype) -> dict:
 
 def pack_rglru(spec: RGLRUSpec, t: dict, device, act_dtype) -> dict:
     """t: y, y.b, x, x.b, conv, conv.b, ra, ra.b, ri, ri.b, lam, o.  y | x are one biased projection; the two gate
-    matrices of a block become one float32 [blocks, in, 2 out] operand; softplus(lam) is formed once, in float32."""
+    matrices of a block become one [blocks, in, 2 out] operand (its product accumulates and lands in float32);
+    softplus(lam) is formed once, in float32."""
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
     f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
     wg = torch.cat([t["ra"].float().transpose(1, 2), t["ri"].float().transpose(1, 2)], 2)
     bg = torch.cat([t["ra.b"].float(), t["ri.b"].float()], 1)[:, None, :]
     return dict(w_yx=a(torch.cat([t["y"], t["x"]], 0)), b_yx=a(torch.cat([t["y.b"], t["x.b"]], 0)), taps=f(t["conv"]),
-                b_conv=f(t["conv.b"]), w_gates=f(wg), b_gates=f(bg),
+                b_conv=f(t["conv.b"]), w_gates=a(wg), b_gates=f(bg),
                 sp=f(torch.nn.functional.softplus(t["lam"].float(), threshold=30.0)), w_o=a(t["o"]))
 
 

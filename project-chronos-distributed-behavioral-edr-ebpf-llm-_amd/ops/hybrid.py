@@ -276,11 +276,15 @@ def gated_group_norm(o, skip_src, skip_off: int, skip_w, gate_src, g_off: int, w
 
 def block_gates(u, w_gates, b_gates):
     """Gate pre-activations of a block-diagonal projection, float32: u [T, W] split into NB blocks of channels, block b
-    times w_gates[b] ([W / NB, n]) plus b_gates[b] ([1, n]).  Returns [NB, T, n].  A float32 library product on both
-    devices and in both activation dtypes (its outputs are gates of a recurrence)."""
+    times w_gates[b] ([W / NB, n]) plus b_gates[b] ([1, n], float32).  Returns [NB, T, n].  A library product with
+    float32 accumulation and float32 output (its results are gates of a recurrence): bfloat16 operands go to the
+    matrix cores as they are (their products are exact in float32), float32 operands to the float32 GEMM."""
     NB = w_gates.shape[0]
     T, W = u.shape
-    return torch.baddbmm(b_gates, u.float().view(T, NB, W // NB).transpose(0, 1), w_gates)
+    ub = u.view(T, NB, W // NB).transpose(0, 1)
+    if u.is_cuda and u.dtype == torch.bfloat16 and w_gates.dtype == torch.bfloat16:
+        return torch.baddbmm(b_gates, ub, w_gates, out_dtype=torch.float32)
+    return torch.baddbmm(b_gates, ub.float(), w_gates.float())
 
 
 def rglru_scan(u, gates, sp, c: float, ysrc, y_off: int, q_start, pos0, slots, S, act_dtype, max_q: int = 0):

@@ -1,10 +1,13 @@
-"""Throughput of a hybrid design (Zokunex, Kalesun) beside the framework's other models at equal width and depth:
+"""Throughput of a hybrid design (Zokunex, Kalesun, Tugovik) beside the framework's other models at equal width and depth:
 whole-model prefill and decode steps, and each of the design's kernels beside its closest existing kernel with the
 fraction of its roofline it reaches.
 
-``python bench.py --design-compare [--design zokunex|kalesun] [--design-sizes 1k,2k,4k]`` prints one JSON line (the
-default benchmark and its output line are untouched).  Zokunex stands beside Llama; Kalesun beside Zokunex (the
-closest family: recurrent layers, attention and mixtures of experts on a float32 stream) and Llama.  Weights are random; every number is measured on the GPU this process runs on.
+``python bench.py --design-compare [--design zokunex|kalesun|tugovik] [--design-sizes 1k,2k,4k]`` prints one JSON line
+(the default benchmark and its output line are untouched).  Zokunex stands beside Llama; Kalesun beside Zokunex (the
+closest family: recurrent layers, attention and mixtures of experts on a float32 stream) and Llama; Tugovik beside
+Kalesun (masked grouped-query attention over paged keys and values, linear-state scans behind a short convolution,
+gated experts, RMS norms on the stream) and Llama.  Weights are random; every number is measured on the GPU this
+process runs on.
 
 Rooflines: HBM 8 TB/s for kernels bound by the bytes they must move, 2.5 PFLOP/s dense bf16 for the matrix-shaped
 ones (the attention kernels over a long context are priced by their FLOPs in prefill and by their cache bytes in
@@ -70,6 +73,29 @@ def kalesun_config(size: dict) -> dict:
     layers = [dict(mix_d, mlp=dense), dict(mix_a, mlp=moe), dict(mix_g, mlp=moe), dict(mix_a, mlp=dense)][:LAYERS]
     return dict(architecture="Kalesun", vocab=VOCAB, width=size["width"], postln_alpha=2.0, norm=dict(eps=1e-6),
                 layers=layers)
+
+# Tugovik: width -> (attention heads, kv heads, dim, vdim, chunk | state-space heads, vdim, state, groups |
+#                    recurrence width, blocks | experts, top, groups, kept, expert ff, shared ff | token-input columns)
+TUGOVIK_SIZES = {
+    "1k": dict(width=1024, a=(8, 2, 128, 128, 512), m=(32, 64, 128, 4), r=(1024, 4), moe=(8, 2, 4, 2, 512, 1024), side=128),
+    "2k": dict(width=2048, a=(16, 4, 128, 128, 1024), m=(64, 64, 128, 8), r=(2048, 8), moe=(16, 4, 4, 2, 1024, 2048), side=256),
+    "4k": dict(width=4096, a=(32, 8, 128, 128, 1024), m=(128, 64, 128, 8), r=(4096, 16), moe=(32, 4, 8, 4, 1536, 4096), side=256),
+}
+
+
+def tugovik_config(size: dict) -> dict:
+    ah, ag, ad, av, chunk = size["a"]
+    mh, mv, mn, mg = size["m"]
+    rw, rb = size["r"]
+    ne, top, ng, keep, eff, sff = size["moe"]
+    mix_a = dict(type="attention", mixer=dict(heads=ah, kv_heads=ag, dim=ad, vdim=av, scale=ad ** -0.5, mask=dict(size=chunk)))
+    mix_m = dict(type="mamba2", mixer=dict(heads=mh, vdim=mv, state=mn, groups=mg, conv=4, norm_groups=mg))
+    mix_r = dict(type="rglru", mixer=dict(width=rw, blocks=rb, conv=4))
+    moe = dict(kind="moe", expert=dict(ff=eff), shared=dict(ff=sff),
+               router=dict(experts=ne, top=top, scale=2.5, groups=dict(count=ng, keep=keep)))
+    layers = [dict(mix_m, mlp=moe), dict(mix_a, mlp=moe), dict(mix_r, mlp=moe), dict(mix_a, mlp=moe)][:LAYERS]
+    return dict(architecture="Tugovik", vocab=VOCAB, width=size["width"], norm=dict(eps=1e-6), layers=layers,
+                token_side=dict(dim=size["side"]))
 
 
 def _say(msg: str) -> None:
@@ -359,6 +385,216 @@ def _kernels_kalesun(size: dict, zsize: dict, dev, T: int, ctx: int, rows: int) 
     return out
 
 
+def _kernels_tugovik(size: dict, ksize: dict, dev, T: int, ctx: int, rows: int) -> dict:
+    """Tugovik's kernels and their closest existing kernels at this size: seconds, and the fraction of the roofline
+    reached.  ``ksize``: the Kalesun sizes of the same width (for the kernels it stands beside)."""
+    from chronos import ops
+    from chronos.ops import hybrid as hops
+
+    out = {}
+    bf = torch.bfloat16
+    d = size["width"]
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *s, dt=bf, sc=1.0: (torch.randn(*s, device=dev, generator=g) * sc).to(dt)  # noqa: E731
+    i32 = dict(dtype=torch.int32, device=dev)
+
+    def rec(name, secs, nbytes=0.0, flops=0.0):
+        roof = max(nbytes / HBM_BPS, flops / BF16_FLOPS)
+        _say(f"  {name}: {secs * 1e6:.1f} us, roofline {roof * 1e6:.2f} us")
+        out[name] = dict(us=round(secs * 1e6, 1), roofline_us=round(roof * 1e6, 2), of_roofline=round(roof / secs, 4))
+
+    bs = 16
+    seqs = max(1, T // ctx)
+    per = ctx // bs + 1
+    nb = max(seqs, rows) * per + 1
+    bt = torch.arange(1, 1 + seqs * per, **i32).view(seqs, per)
+    qs = torch.arange(0, (seqs + 1) * ctx, ctx, **i32)
+    pos = torch.arange(ctx, **i32).repeat(seqs)
+    tseq = torch.arange(seqs, **i32).repeat_interleave(ctx)
+    btd = torch.arange(1, 1 + rows * per, **i32).view(rows, per)
+    qsd = torch.arange(rows + 1, **i32)
+    posd = torch.full((rows,), ctx, **i32)
+    tseqd = torch.arange(rows, **i32)
+    NS = max(seqs, rows) + 1
+    p0, sl, sld = torch.zeros(seqs, **i32), torch.arange(seqs, **i32), torch.arange(rows, **i32)
+    # ---- the stream's joins
+    y, y2, x32, w32 = rnd(T, d), rnd(T, d), rnd(T, d, dt=torch.float32), rnd(d, dt=torch.float32)
+    g2 = rnd(T, 1, dt=torch.float32)
+    rec("add_rms_norm", _time(lambda: hops.add_rms_norm(y, x32, w32, 1e-6, bf)), T * d * (2 + 4 + 4 + 2))
+    rec("add_rms_norm.gated_pair", _time(lambda: hops.add_rms_norm(y, x32, None, 1e-6, bf, y2, g2)), T * d * (2 + 2 + 4 + 4 + 2))
+    rec("add_rms_norm.normed_addend", _time(lambda: hops.add_rms_norm(y, x32, w32, 1e-6, bf, w_y=w32)), T * d * (2 + 4 + 4 + 2))
+    rec("kalesun.scale_add_rms_norm", _time(lambda: hops.scale_add_rms_norm(y, x32, w32, 1.0, 1e-6, bf)), T * d * (2 + 4 + 4 + 2))
+    xb, wb = rnd(T, d), rnd(d)
+    rec("llama.add_rmsnorm", _time(lambda: ops.add_rmsnorm(y, xb, wb, 1e-5)), T * d * (2 + 2 + 2 + 2))
+    sd = size["side"]
+    a_, table, ids = rnd(T, sd), rnd(VOCAB, 4 * sd), torch.randint(0, VOCAB, (T,), device=dev, generator=g).int()
+    rec("token_gate", _time(lambda: hops.token_gate(a_, ids, table, sd, bf)), T * sd * 6.0)
+    # ---- attention: the chunk mask beside Kalesun's window of the same span (with sink and gate) and Llama's
+    H, G, D, Dv, chunk = size["a"]
+    kc, vc = rnd(nb, bs, G, D, sc=0.3), rnd(nb, bs, G, Dv, sc=0.3)
+    C = (H + G) * D + G * Dv
+    qkv = rnd(seqs * ctx, C, sc=0.3)
+    vis = sum(i % chunk + 1 for i in range(ctx))
+    rec("chunk_attention.prefill", _time(lambda: hops.window_attention(qkv, kc, vc, bt, qs, pos, None, None, D ** -0.5, 0, 0, H, bf, ctx, chunk), iters=3, warm=1),
+        flops=2.0 * seqs * vis * H * (D + Dv))
+    rec("window_prep.plain.prefill", _time(lambda: hops.window_prep(qkv, H, G, D, Dv, None, None, pos, tseq, bt, None, None, 1e-6, None, 0, kc, vc, False)),
+        nbytes=seqs * ctx * 2 * G * (D + Dv) * 2.0)
+    qkvd = rnd(rows, C, sc=0.3)
+    rec("chunk_attention.decode", _time(lambda: hops.window_attention(qkvd, kc, vc, btd, qsd, posd, None, None, D ** -0.5, 0, 0, H, bf, 1, chunk)),
+        nbytes=rows * (ctx % chunk + 1) * G * (D + Dv) * 2.0)
+    posm = torch.full((rows,), ctx // chunk * chunk + chunk - 1, **i32)   # the last position of a chunk: every key of it
+    btm = torch.arange(1, 1 + rows * (per + chunk // bs), **i32).view(rows, -1) % (nb - 1) + 1
+    rec("chunk_attention.decode_full_chunk", _time(lambda: hops.window_attention(qkvd, kc, vc, btm, qsd, posm, None, None, D ** -0.5, 0, 0, H, bf, 1, chunk)),
+        nbytes=rows * chunk * G * (D + Dv) * 2.0)
+    kH, kG, kD, kDv, win, keep = ksize["a"]
+    kkc, kvc = rnd(nb, bs, kG, kD, sc=0.3), rnd(nb, bs, kG, kDv, sc=0.3)
+    kqkv = rnd(seqs * ctx, (kH + kG) * kD + kG * kDv, sc=0.3)
+    kgate, ksink = rnd(seqs * ctx, kH, dt=torch.float32), rnd(kH, dt=torch.float32)
+    kvis = sum(min(i + 1, win) + max(0, min(keep, i + 1 - win)) for i in range(ctx))
+    rec("kalesun.window_attention.prefill", _time(lambda: hops.window_attention(kqkv, kkc, kvc, bt, qs, pos, ksink, kgate, kD ** -0.5, win, keep, kH, bf, ctx), iters=3, warm=1),
+        flops=2.0 * seqs * kvis * kH * (kD + kDv))
+    kqkvd, kgated = rnd(rows, (kH + kG) * kD + kG * kDv, sc=0.3), rnd(rows, kH, dt=torch.float32)
+    rec("kalesun.window_attention.decode", _time(lambda: hops.window_attention(kqkvd, kkc, kvc, btd, qsd, posd, ksink, kgated, kD ** -0.5, win, keep, kH, bf, 1)),
+        nbytes=rows * (min(ctx + 1, win) + keep) * kG * (kD + kDv) * 2.0)
+    hq = d // 128
+    hkv = max(1, hq // 4)
+    lkc, lvc = rnd(nb, hkv, bs, 128, sc=0.3), rnd(nb, hkv, 128, bs, sc=0.3)
+    q = rnd(seqs * ctx, hq, 128, sc=0.3)
+    ctxl = torch.full((seqs,), ctx, **i32)
+    tiles = torch.tensor(ops.attention_tiles([ctx] * seqs, hq, hkv, 8), **i32).view(-1, 2)
+    rec("llama.attention.prefill", _time(lambda: ops.paged_attention(q, lkc, lvc, bt, qs, ctxl, tiles, tiles.shape[0], 8, 1), iters=3, warm=1),
+        flops=4.0 * seqs * ctx * (ctx + 1) / 2 * hq * 128)
+    qd = rnd(rows, hq, 128, sc=0.3)
+    ctxd = torch.full((rows,), ctx + 1, **i32)
+    ns = ops.pick_nsplit(rows * hkv, ctx + 1)
+    rec("llama.attention.decode", _time(lambda: ops.paged_attention(qd, lkc, lvc, btd, qsd, ctxd, None, rows, 1, ns)),
+        nbytes=rows * (ctx + 1) * hkv * 128 * 2 * 2.0)
+    # ---- the state-space layer: convolution, per-token scalars, scan, gated group norm
+    mh, mv, mn, mg = size["m"]
+    inner, Cc = mh * mv, mh * mv + 2 * mg * mn
+    proj, taps, cb = rnd(seqs * ctx, inner + Cc, sc=0.5), rnd(Cc, 4, dt=torch.float32), rnd(Cc, dt=torch.float32)
+    hist = torch.zeros(NS, 3, Cc, device=dev, dtype=bf)
+    rec("short_conv.bias.prefill", _time(lambda: hops.short_conv(proj, taps, tseq, qs, p0, sl, hist, True, cb, inner)),
+        nbytes=seqs * ctx * Cc * 4.0)
+    xbc = hops.short_conv(proj, taps, tseq, qs, p0, sl, hist, True, cb, inner)
+    dtp, alog = rnd(seqs * ctx, mh, dt=torch.float32), rnd(mh, dt=torch.float32, sc=0.3)
+    rec("ssm_prep.prefill", _time(lambda: hops.ssm_prep(dtp, alog)), nbytes=seqs * ctx * mh * 12.0)
+    decay, dts = hops.ssm_prep(dtp, alog)
+    S = torch.zeros(NS, mh, mn, mv, device=dev)
+    rec("linear_scan.ssm.prefill", _time(lambda: hops.linear_scan(xbc, inner + mg * mn, inner, 0, None, None, 1.0, decay, None, qs, p0, sl, S, mg, mh, mn, mv, dts), iters=3, warm=1),
+        nbytes=seqs * ctx * Cc * 2.0, flops=seqs * ctx * mh * mn * mv * 4.0)
+    xbcd = rnd(rows, Cc, sc=0.5)
+    decd, dtd = torch.rand(rows, mh, device=dev), torch.rand(rows, mh, device=dev)
+    rec("linear_scan.ssm.decode", _time(lambda: hops.linear_scan(xbcd, inner + mg * mn, inner, 0, None, None, 1.0, decd, None, qsd, posd, sld, S, mg, mh, mn, mv, dtd)),
+        nbytes=rows * mh * mn * mv * 4 * 2.0)
+    o = torch.randn(seqs * ctx, mh, mv, device=dev)
+    skip, nw = rnd(mh, dt=torch.float32), rnd(inner, dt=torch.float32)
+    rec("gated_group_norm.prefill", _time(lambda: hops.gated_group_norm(o, xbc, 0, skip, proj, 0, nw, mg, 1e-6, bf)),
+        nbytes=seqs * ctx * inner * (4 + 2 + 2 + 2.0))
+    rec("kalesun.head_norm_gate.prefill", _time(lambda: hops.head_norm_gate(o, proj, 0, nw, 1e-6, True, bf)),
+        nbytes=seqs * ctx * inner * (4 + 2 + 2.0))
+    for name, (hh, hk, dd, dv), delta in (("delta", ksize["d"], True), ("gla", (ksize["g"][0], ksize["g"][0], *ksize["g"][1:]), False)):
+        Cq = 2 * hk * dd + hh * dv
+        kS = torch.zeros(NS, hh, dd, dv, device=dev)
+
+        def scan(pr, qs_, p0_, sl_, n):
+            if delta:
+                qsc, ksc = torch.rand(n, hk, device=dev), torch.rand(n, hk, device=dev)
+                dec, beta = torch.rand(n, hh, device=dev), torch.rand(n, hh, device=dev)
+                return lambda: hops.linear_scan(pr, 0, hk * dd, 2 * hk * dd, qsc, ksc, 1.0, dec, beta, qs_, p0_, sl_, kS, hk, hh, dd, dv)
+            dec = torch.rand(n, hh, dd, device=dev)
+            return lambda: hops.linear_scan(pr, 0, hk * dd, 2 * hk * dd, None, None, dd ** -0.5, dec, None, qs_, p0_, sl_, kS, hk, hh, dd, dv)
+
+        kp = rnd(seqs * ctx, Cq, sc=0.5)
+        rec(f"kalesun.linear_scan.{name}.prefill", _time(scan(kp, qs, p0, sl, seqs * ctx), iters=3, warm=1),
+            nbytes=seqs * ctx * Cq * 2.0, flops=seqs * ctx * hh * dd * dv * (6.0 if delta else 4.0))
+        kpd = rnd(rows, Cq, sc=0.5)
+        rec(f"kalesun.linear_scan.{name}.decode", _time(scan(kpd, qsd, posd, sld, rows)), nbytes=rows * hh * dd * dv * 4 * 2.0)
+    # ---- the gated linear recurrence: block-diagonal gate projections (float32 library product) and the scan
+    rw, rb = size["r"]
+    bw = rw // rb
+    yx = rnd(seqs * ctx, 2 * rw, sc=0.5)
+    u = rnd(seqs * ctx, rw, sc=0.5)
+    wg, bg = rnd(rb, bw, 2 * bw, sc=bw ** -0.5), rnd(rb, 1, 2 * bw, dt=torch.float32)   # bfloat16 weights, float32 out
+    rec("block_gates.prefill", _time(lambda: hops.block_gates(u, wg, bg), iters=3, warm=1),
+        nbytes=seqs * ctx * rw * (2 + 8.0), flops=seqs * ctx * rw * bw * 4.0)
+    gates = hops.block_gates(u, wg, bg)
+    sp = torch.rand(rw, device=dev)
+    Sr = torch.zeros(NS, rw, device=dev)
+    rec("rglru_scan.prefill", _time(lambda: hops.rglru_scan(u, gates, sp, 8.0, yx, 0, qs, p0, sl, Sr, bf, ctx), iters=3, warm=1),
+        nbytes=seqs * ctx * rw * (8 + 2 + 2 + 2.0))
+    ud, yxd = rnd(rows, rw, sc=0.5), rnd(rows, 2 * rw, sc=0.5)
+    rec("block_gates.decode", _time(lambda: hops.block_gates(ud, wg, bg)), nbytes=rb * bw * 2 * bw * 4.0)
+    gd = hops.block_gates(ud, wg, bg)
+    rec("rglru_scan.decode", _time(lambda: hops.rglru_scan(ud, gd, sp, 8.0, yxd, 0, qsd, posd, sld, Sr, bf, 1)),
+        nbytes=rows * rw * (8 + 2 + 2 + 2 + 8.0))
+    # ---- feed-forwards: the grouped sigmoid router beside the top-k softmax router; the experts are Kalesun's kernel
+    ne, top, ng, keep, eff, sff = size["moe"]
+    wr, br = rnd(ne, d, sc=0.05), rnd(ne, dt=torch.float32, sc=0.01)
+    wgu = rnd(ne, 2 * eff, d, sc=d ** -0.5)[:, hops.moe_glu_row_order(eff).to(dev)].contiguous()
+    wd = rnd(ne, d, eff, sc=eff ** -0.5)
+    inf = float("inf")
+    for name, tk in (("prefill", T), ("decode", rows)):
+        h = rnd(tk, d)
+        rec(f"moe_route_group.{name}", _time(lambda: hops.moe_route_group(h, wr, top, ng, keep, 2.5)), nbytes=tk * d * 2.0 + ne * d * 2.0)
+        rec(f"kalesun.moe_route_topk.{name}", _time(lambda: hops.moe_route_topk(h, wr, br, top)), nbytes=tk * d * 2.0 + ne * d * 2.0)
+        idx, wt = hops.moe_route_group(h, wr, top, ng, keep, 2.5)
+        used = min(ne, tk * top) * 3 * eff * d * 2.0
+        rec(f"moe_glu_ffn.silu.{name}", _time(lambda: hops.moe_glu_ffn(h, idx, wt, wgu, wd, inf, 1.0, 0.0, bf, True), iters=3, warm=1),
+            nbytes=used + tk * d * 4.0, flops=tk * top * 6.0 * eff * d)
+        rec(f"kalesun.moe_glu_ffn.{name}", _time(lambda: hops.moe_glu_ffn(h, idx, wt, wgu, wd, 7.0, 1.702, 1.0, bf, True), iters=3, warm=1),
+            nbytes=used + tk * d * 4.0, flops=tk * top * 6.0 * eff * d)
+        lf = int(3.5 * d)
+        wgl, wdn = rnd(2 * lf, d, sc=d ** -0.5), rnd(d, lf, sc=lf ** -0.5)
+        rec(f"llama.mlp.{name}", _time(lambda: ops.linear(ops.gate_up_silu(h, wgl), wdn), iters=3, warm=1),
+            nbytes=3 * lf * d * 2.0 + tk * d * 4.0, flops=tk * 6.0 * lf * d)
+    return out
+
+
+def run_tugovik(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int = 2048, device: str = "cuda") -> dict:
+    from chronos import ops
+    from chronos.models import kalesun, llama, tugovik
+    from chronos.models.hybrid import HybridDecoder
+
+    dev = torch.device(device if ":" in device else device + ":0")
+    torch.cuda.set_device(dev)
+    ops.load()
+    ops.device_init()
+    res = {}
+    P = ctx + plen + 16
+    for name in sizes:
+        size, ksize = TUGOVIK_SIZES[name], KALESUN_SIZES[name]
+        t0 = time.time()
+        cfg = tugovik.config_from_dict(tugovik_config(size), name=f"tugovik-{name}", max_position=P)
+        tm = HybridDecoder(cfg, tugovik.pack_weights(cfg, tugovik.random_tensors(cfg, 0), dev, torch.bfloat16), dev, P,
+                           torch.bfloat16)
+        entry = dict(tugovik=dict(params=cfg.param_count(), **_model_steps(tm, dev, seqs, plen, rows, ctx)))
+        _say(f"size {name}: tugovik {entry['tugovik']}")
+        del tm
+        kcfg = kalesun.config_from_dict(kalesun_config(ksize), name=f"kalesun-{name}", max_position=P)
+        km = HybridDecoder(kcfg, kalesun.pack_weights(kcfg, kalesun.random_tensors(kcfg, 0), dev, torch.bfloat16), dev, P,
+                           torch.bfloat16)
+        entry["kalesun"] = dict(params=kcfg.param_count(), **_model_steps(km, dev, seqs, plen, rows, ctx))
+        _say(f"  kalesun {entry['kalesun']}")
+        del km
+        d = size["width"]
+        lc = llama.LlamaConfig(name=f"llama-{name}", vocab_size=VOCAB, hidden_size=d, intermediate_size=int(3.5 * d),
+                               num_layers=LAYERS, num_heads=d // 128, num_kv_heads=max(1, d // 512), max_position=P)
+        lm = llama.LlamaModel(lc, llama.random_weights(lc, None, dev, 0), None, dev, P)
+        entry["llama"] = dict(params=lc.param_count(), **_model_steps(lm, dev, seqs, plen, rows, ctx))
+        _say(f"  llama {entry['llama']}")
+        del lm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _kernels_tugovik(size, ksize, dev, seqs * plen, ctx, rows)
+        entry["seconds"] = round(time.time() - t0, 1)
+        res[name] = entry
+        torch.cuda.empty_cache()
+    return dict(metric="design_compare", design="tugovik", beside="kalesun and llama (equal width and depth)",
+                layers=LAYERS, workload=dict(prefill=f"{seqs} x {plen} tokens in one step",
+                                             decode=f"{rows} rows at context {ctx}"),
+                dtype="bf16", data="synthetic", sizes=res)
+
+
 def run_kalesun(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int = 2048, device: str = "cuda") -> dict:
     from chronos import ops
     from chronos.models import kalesun, llama, zokunex
@@ -441,6 +677,7 @@ def run(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int =
 
 def main(a) -> int:
     sizes = [s for s in a.design_sizes.split(",") if s]
-    out = (run_kalesun if getattr(a, "design", "zokunex") == "kalesun" else run)(sizes, device=a.device)
+    fn = {"kalesun": run_kalesun, "tugovik": run_tugovik}.get(getattr(a, "design", "zokunex"), run)
+    out = fn(sizes, device=a.device)
     print(json.dumps(out), flush=True)
     return 0
