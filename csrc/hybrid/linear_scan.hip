@@ -1,9 +1,10 @@
 // linear_scan.hip — recurrent mixers whose per-head state is a D x Dv matrix updated by rank-one writes: the gated
 // delta rule and gated linear attention, plus the short causal convolution and the per-token scalars that feed them.
 //
-//   short_conv    y[t, c] = act(bias[c] + sum_i w[c, i] x[t - (K-1) + i, c]) over each sequence's own tokens; inputs before the
-//                 step's first token come from the sequence's history rows (its last K-1 inputs, by state slot), or
-//                 are zero when the step starts at position 0.  A second launch then rewrites the history.
+//   short_conv    y[t, c] = act(bias[c] + sum_i w[c, i] x[t - (K-1) + i, c]) over each sequence's own tokens (the
+//                 bias is optional); inputs before the step's first token come from the sequence's history rows (its
+//                 last K-1 inputs, by state slot), or are zero when the step starts at position 0.  A second launch
+//                 then rewrites the history.
 //   delta_prep    per token: 1 / |q|, 1 / |k| per query/key head (float), decay = exp(-exp(A) softplus(a)) and
 //                 beta = sigmoid(b) per value head.
 //   linear_scan   per (sequence, value head, 64 value columns): the state lives in registers (a wave owns 16 columns,
@@ -112,7 +113,8 @@ template <> __device__ __forceinline__ uint16_t zero_of<uint16_t>() { return 0; 
 
 // 256 threads: wave w owns 64 / RG value columns of the workgroup's 4 x 64 / RG; a lane holds DP / RG rows of one
 // column.  LDS (floats): q [TC][DP] | k [TC][DP] | (CHD: decay rows [TC][DP]) | v [TC][64] | per token: decay, beta,
-// q scale, k scale (times the value's per-head scale when one is given).  The next stage's global loads are issued before the current stage's tokens are processed and
+// q scale, k scale (times the value's per-head scale when one is given).  The next stage's global loads are issued
+// before the current stage's tokens are processed and
 // land in LDS afterwards, so the token loop never waits on global memory; the scales of q and k are folded into
 // per-token scalars (S^T k_hat = s_k S^T k, k_hat u^T = k (s_k u)^T, S^T q_hat = s_q S^T q).
 // PIPE: the one-pass token loops with LDS rows prefetched (more registers: for launches with prompt portions);
@@ -419,7 +421,8 @@ static bool linear_scan_d(bool pipe, const T* proj, int ldp, int q_off, int k_of
     return true;
 }
 
-// delta: beta != nullptr.  vscale (float [T, H], may be nullptr; without delta only): a factor on the written value.  chd: decay holds one number per state row ([T, H, D]) instead of one per head ([T, H]).
+// delta: beta != nullptr.  vscale (float [T, H], may be nullptr; without delta only): a factor on the written value.
+// chd: decay holds one number per state row ([T, H, D]) instead of one per head ([T, H]).
 // Returns false when D has no instantiation (D > 256).
 bool launch_hy_linear_scan(const void* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
                            const float* kscale, float q_mul, const float* decay, bool chd, const float* beta,

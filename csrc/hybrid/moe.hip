@@ -4,8 +4,8 @@
 //           hybrid_elementwise.hip), then one wave per token: softmax over all N, the `top` largest
 //           of score + correction chosen (the correction steers the choice only), weights = the chosen outputs' plain
 //           scores, not renormalised.  Ties go to the lower index.
-//   route_group  sigmoid scores; the outputs form equal groups of neighbours, a group scores the sum of its two
-//           largest scores, only the best `keep` groups stay eligible, the `top` largest eligible scores are chosen and
+//   route_group  sigmoid scores; the outputs form equal groups of neighbours, a group scores its top two
+//           scores added up, only the best `keep` groups stay eligible, the `top` largest eligible scores are chosen and
 //           weighted by score / (sum of the chosen + 1e-20) * scale.
 //   ffn     per token: sum over its chosen experts of weight * W_down act(W_up h); an index >= E is an identity
 //           expert (weight * h).  Token-parallel form: one workgroup per token streams the chosen experts' weights
@@ -170,7 +170,7 @@ __global__ void __launch_bounds__(256) moe_select_topk_kernel(const float* __res
 }
 
 // One wave per token: sigmoid scores of z [T, N], the choice limited to the best groups (ng groups of N / ng
-// neighbouring outputs, a group's score = the sum of its two largest scores, the `keep` best stay; ties: the lower
+// neighbouring outputs, a group's score = its top two scores added up, the `keep` best stay; ties: the lower
 // index), then the `top` largest eligible scores (ties: the lower index), weights = score / (their sum + 1e-20) * scale.
 // ng <= 64 (lane g ranks group g), top <= 64 (lane k keeps the k-th choice).  LDS per wave: N scores, ng flags.
 __global__ void __launch_bounds__(256) moe_select_group_kernel(const float* __restrict__ z, int32_t* __restrict__ idx,

@@ -1,10 +1,11 @@
 // window_attention.hip — grouped-query softmax attention over paged keys and values through a sliding window that
 // also keeps each sequence's first tokens, with a learned sink per head in the softmax denominator.
 //
-//   window_prep       per token: per-head RMS norm (float; skipped when no norm weights are given) and rotation (cos / sin from a float table made in double
-//                     precision) of the query heads (in place) and key heads; the values optionally mixed with the
-//                     same token's values of an earlier layer, (1 - lam) v + lam v_first; keys and values written to
-//                     the token's page and slot of kc [NB, BS, G, D] / vc [NB, BS, G, Dv].
+//   window_prep       per token: per-head RMS norm (float; skipped when no norm weights are given) and rotation
+//                     (cos / sin from a float table made in double precision) of the query heads (in place) and key
+//                     heads; the values optionally mixed with the same token's values of an earlier layer,
+//                     (1 - lam) v + lam v_first; keys and values written to the token's page and slot of
+//                     kc [NB, BS, G, D] / vc [NB, BS, G, Dv].
 //   window_attention  the general kernel (vector ALUs, float or bfloat16, any sizes): a workgroup takes one sequence,
 //                     one key/value head and up to 16 consecutive query tokens with all the query heads of that
 //                     group (at most 64 (token, head) rows, fewer when the LDS asks for it); 64-key tiles of the

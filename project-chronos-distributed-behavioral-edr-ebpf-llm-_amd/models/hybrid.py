@@ -3,8 +3,8 @@ attention, windowed or chunked attention, gated delta rule, gated linear attenti
 linear recurrence) and an optional feed-forward (dense, gated, mixture of experts), on a float32 residual stream.
 The stream's rule is a parameter of the configuration: the norm on the sublayer's OUTPUT (``out_norm``:
 x <- x + layer_norm(sublayer(x))), AFTER the sum (``post_norm``: x <- rms_norm(alpha x + sublayer(x))) or on the
-sublayer's INPUT (``pre_norm``: x <- x + sublayer(rms_norm(x))).  A range of layers may run several times in a row
-with the same weights (``loop``); every run has its own pages and state.
+sublayer's INPUT (``pre_norm``: x <- x + sublayer(rms_norm(x))).  A range of layers may repeat, back to back, on
+shared weights (``loop``); every run has its own pages and state.
 
 This module is the design-independent part: the mixer and feed-forward kinds with their sizes and constants as
 parameters, the cache that holds pages for the attention layers and state slots for the recurrent ones, and the
@@ -140,7 +140,7 @@ class GLASpec:
 class Mamba2Spec:
     """State-space duality: per head a state x vdim matrix S <- exp(-exp(A) dt) S + dt B x^T, read by C, with B and C
     shared by the heads of a group; x, B and C pass a short causal convolution (with bias) and SiLU; the read-out
-    plus D x is gated by silu(z) and then RMS-normed in ``norm_groups`` equal parts."""
+    plus D x is gated by silu(z) first and RMS-normed afterwards, over ``norm_groups`` column ranges of equal size."""
     heads: int
     vdim: int
     state: int
@@ -158,8 +158,8 @@ class Mamba2Spec:
         return self.inner + 2 * self.groups * self.state
 
     def params(self, d: int) -> int:
-        return d * (2 * self.inner + 2 * self.groups * self.state + self.heads) + self.conv_channels * (self.conv + 1) + \
-            3 * self.heads + self.inner + self.inner * d
+        n_in = 2 * self.inner + 2 * self.groups * self.state + self.heads
+        return d * n_in + self.conv_channels * (self.conv + 1) + 3 * self.heads + self.inner + self.inner * d
 
 
 @dataclass
@@ -175,8 +175,8 @@ class RGLRUSpec:
 
     def params(self, d: int) -> int:
         bw = self.width // self.blocks
-        return 2 * self.width * (d + 1) + self.width * (self.conv + 1) + 2 * self.blocks * bw * (bw + 1) + self.width + \
-            self.width * d
+        gates = 2 * self.blocks * bw * (bw + 1)
+        return 2 * self.width * (d + 1) + self.width * (self.conv + 1) + gates + self.width + self.width * d
 
 
 @dataclass
@@ -206,7 +206,7 @@ class MoEGluSpec:
 @dataclass
 class MoEGroupGluSpec:
     """Mixture of gated experts behind a sigmoid router whose choice is limited to the best groups of neighbouring
-    experts (a group scores the sum of its two largest scores); weights = chosen scores / their sum * scale.  With
+    experts (a group scores its top two scores added up); weights = chosen scores / their sum * scale.  With
     ``shared_ff`` > 0 a shared gated expert of that size runs for every token, times sigmoid of one more projection."""
     experts: int
     top: int
@@ -241,7 +241,7 @@ class HybridConfig:
     #                                "pre_norm": x <- x + sublayer(rms_norm(x))
     residual_alpha: float = 1.0
     tied_head: bool = False        # the logits come from the embedding table
-    loop: Optional[tuple] = None   # (start, stop, times): layers start .. stop-1 run ``times`` times in a row
+    loop: Optional[tuple] = None   # (start, stop, times): layers [start, stop) run ``times`` times, back to back
     token_side: int = 0            # > 0: after every layer's feed-forward a gated, RMS-normed projection of this many
     #                                columns of a second embedding table (layer i owns columns [i dim, (i+1) dim))
 
@@ -447,8 +447,8 @@ def pack_mamba2(spec: Mamba2Spec, t: dict, device, act_dtype) -> dict:
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
     f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
     n = 2 * spec.inner + 2 * spec.groups * spec.state
-    return dict(w_in=a(t["in"][:n]), w_dt=a(t["in"][n:]), b_dt=f(t["dt_bias"]), taps=f(t["conv"]), b_conv=f(t["conv.b"]),
-                a_log=f(t["A_log"]), skip=f(t["D"]), norm=f(t["norm"]), w_o=a(t["o"]))
+    return dict(w_in=a(t["in"][:n]), w_dt=a(t["in"][n:]), b_dt=f(t["dt_bias"]), taps=f(t["conv"]),
+                b_conv=f(t["conv.b"]), a_log=f(t["A_log"]), skip=f(t["D"]), norm=f(t["norm"]), w_o=a(t["o"]))
 
 
 def pack_rglru(spec: RGLRUSpec, t: dict, device, act_dtype) -> dict:

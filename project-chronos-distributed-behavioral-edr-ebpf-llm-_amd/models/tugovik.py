@@ -3,7 +3,7 @@ tokens with chunked grouped-query attention (biased projections, no rotation, ke
 own chunk of positions), with a state-space-duality layer (Mamba-2) or with a real-gated linear recurrent unit, feed
 forward through a mixture of gated experts behind a sigmoid router whose choice is limited to the best groups of
 experts, plus a shared expert with its own sigmoid gate, and add after every layer a gated projection of the token's
-row in a second embedding table.  A range of layers may run several times in a row with the same weights.
+row in a second embedding table.  A range of layers may repeat, back to back, on shared weights.
 
 This module is the design's reader: ``config.json`` -> :class:`chronos.models.hybrid.HybridConfig`, the checkpoint's
 tensor names -> the packed weights the hybrid kernels take, and random weights of the same shapes for benchmarks and
@@ -99,8 +99,8 @@ def config_to_dict(cfg: HybridConfig) -> dict:
         f = l.ff
         mlp = None
         if f is not None:
-            mlp = dict(kind="moe", expert=dict(ff=f.ff),
-                       router=dict(experts=f.experts, top=f.top, scale=f.scale, groups=dict(count=f.groups, keep=f.keep)))
+            mlp = dict(kind="moe", expert=dict(ff=f.ff), router=dict(experts=f.experts, top=f.top, scale=f.scale,
+                                                                    groups=dict(count=f.groups, keep=f.keep)))
             if f.shared_ff:
                 mlp["shared"] = dict(ff=f.shared_ff)
         layers.append(dict(type=typ, mixer=mixer, mlp=mlp))
@@ -280,7 +280,8 @@ def _preset(width, vocab, pattern, heads, kv_heads, dim, chunk, state, ssm_group
 PRESETS = {
     "tugovik-tiny": _preset(128, 512, "mar", 2, 1, 32, 24, 16, 1, 128, 2, 8, 2, 4, 2, 64, 64, 16, loop=(0, 2, 2)),
     "tugovik-1b": _preset(2048, 32768, "marAmara", 16, 4, 128, 1024, 128, 4, 2048, 8, 16, 4, 4, 2, 1024, 2048, 256),
-    "tugovik-8b-layers": _preset(4096, 128256, "mara", 32, 8, 128, 4096, 128, 8, 4096, 16, 32, 4, 8, 4, 2048, 4096, 256),
+    "tugovik-8b-layers": _preset(4096, 128256, "mara", 32, 8, 128, 4096, 128, 8, 4096, 16, 32, 4, 8, 4, 2048, 4096,
+                                 256),
 }
 
 

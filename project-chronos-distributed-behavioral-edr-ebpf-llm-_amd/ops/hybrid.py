@@ -245,7 +245,7 @@ def moe_glu_ffn(h, idx, wt, w_gu, w_down, limit: float, slope: float, shift: flo
 
 
 def add_rms_norm(y, x, w_out, eps: float, act_dtype, y2=None, gate2=None, w_y=None, emit: bool = True):
-    """x (float32 residual, in place) <- x + v, v = y (+ sigmoid(gate2) y2), divided by its own root mean square and
+    """x (float32 residual, in place) <- x + v, v = y (+ sigmoid(gate2) y2), scaled to unit RMS and
     times w_y when that is given.  Returns in the activation dtype rms_norm(x) * w_out, or the updated rows
     themselves when w_out is None (x itself for float32), or None when ``emit`` is off."""
     if _gpu(x):

@@ -248,8 +248,8 @@ def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, 
                      chunk=0):
     """Causal softmax attention over a paged cache through a sliding window that also keeps a sequence's first
     tokens: the query at position i sees key j <= i when i - j < window or j < keep_first (window 0: every j <= i).
-    ``chunk`` > 0 further hides every key outside the query's own chunk of that many positions, counted from
-    position 0 of the sequence: j is visible only when j // chunk == i // chunk.
+    ``chunk`` > 0 further hides every key outside the query's own chunk of that many positions (the chunk grid
+    is anchored at the sequence's first position): j is visible only when j // chunk == i // chunk.
     ``sink`` f32 [H] or None: exp(sink_h) joins the softmax denominator (no key, no value).  ``gate`` f32 [T, H] or
     None: head h's output times sigmoid(gate).  Queries are the first H D columns of qkv; query head h reads
     key/value head h // (H / G).  Returns [T, H Dv]."""
@@ -421,7 +421,7 @@ def gelu_tanh(z):
 
 def add_rms_norm(y, x, w_out, eps, act_dtype, y2=None, gate2=None, w_y=None, emit=True):
     """The pre-norm stream's join.  v = y (+ sigmoid(gate2) * y2, gate2 f32 [T, 1]); when w_y is given v is first
-    divided by its own root mean square and multiplied by w_y; x (float32, in place) <- x + v.  Returns, in the
+    scaled to unit RMS and multiplied by w_y; x (float32, in place) <- x + v.  Returns, in the
     activation dtype, rms_norm(x) * w_out when w_out is given, else x itself (None when ``emit`` is off)."""
     v = y.float()
     if y2 is not None:
@@ -451,8 +451,8 @@ def ssm_prep(dt_pre, a_log):
 
 def gated_group_norm(o, skip_src, skip_off, skip_w, gate_src, g_off, w, groups, eps, act_dtype):
     """Read-out of a state-space layer: y = (o + skip_w[h] * x) * silu(z) with x = skip_src[:, skip_off:...] and
-    z = gate_src[:, g_off:...] (both [T, H Dv] column ranges), then RMS norm in ``groups`` equal parts of the H Dv
-    columns (each part by its own root mean square), times w [H Dv].  o f32 [T, H, Dv]."""
+    z = gate_src[:, g_off:...] (both [T, H Dv] column ranges), then RMS norm over ``groups`` equal column ranges of the
+    H Dv columns (every range with its own statistic), times w [H Dv].  o f32 [T, H, Dv]."""
     T, H, Dv = o.shape
     n = H * Dv
     y = o + skip_w.float()[None, :, None] * skip_src[:, skip_off:skip_off + n].float().view(T, H, Dv)
@@ -469,7 +469,8 @@ def rglru_scan(u, gates, sp, c, ysrc, y_off, q_start, pos0, slots, S, act_dtype)
         r = sigmoid(gates[.., 0, :]),  i = sigmoid(gates[.., 1, :]),  log a = -c r sp,  a = exp(log a)
         S <- a S + sqrt(1 - a^2) i u;     out = S * gelu_tanh(y)
 
-    u [T, W] (the convolved branch); gates f32 [NB, T, 2 W / NB]: per block of channels the pre-activations of r, then of i;
+    u [T, W] (the convolved branch); gates f32 [NB, T, 2 W / NB]: per block of channels the pre-activations of r,
+    then of i;
     sp f32 [W] = softplus of the decay parameter; y = ysrc[:, y_off : y_off + W]; S f32 [NS, W] by slot, in place; a
     range whose first token sits at position 0 starts from zero.  Returns [T, W] in the activation dtype."""
     T, W = u.shape
@@ -494,7 +495,7 @@ def rglru_scan(u, gates, sp, c, ysrc, y_off, q_start, pos0, slots, S, act_dtype)
 
 def moe_route_group(h, w_router, top, n_groups, keep, scale):
     """Router with sigmoid scores and a choice limited to the best groups: the N outputs form n_groups equal groups
-    of neighbours, a group scores the sum of its two largest scores, the ``keep`` best groups stay, and the ``top``
+    of neighbours, a group scores its top two scores added up, the ``keep`` best groups stay, and the ``top``
     largest scores among them are chosen (ties: the lower index) and weighted by score / (sum of the chosen + 1e-20)
     * scale.  Returns (idx int32 [T, top], weight f32 [T, top])."""
     s = torch.sigmoid(rowdot(h, w_router))

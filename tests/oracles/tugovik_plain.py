@@ -119,7 +119,7 @@ def gated_expert(h, W, p):
 
 
 def route(h, W, p, r):
-    """Chosen experts and their weights: sigmoid scores, the best groups by the sum of their two largest scores, the
+    """Chosen experts and their weights: sigmoid scores, groups ranked by their top two scores added up, the
     largest scores among those groups, normalised and scaled."""
     E, top = r["experts"], r["top"]
     s = sigmoid(W[p + "router"] @ h)
