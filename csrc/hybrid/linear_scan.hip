@@ -388,7 +388,7 @@ static void linear_scan_launch(bool pipe, const T* proj, int ldp, int q_off, int
     if constexpr (HAS_PIPE) {
         const int zp = (Dv + 4 * (64 / hy::kScanRGPrefill) - 1) / (4 * (64 / hy::kScanRGPrefill));
         // The head-decay form without the delta correction serves layers of many narrow heads: once its pipelined
-        // launch (twice the workgroups) no longer fits the chip in one round, the plain loop with half the
+        // launch (twice the workgroups) no longer fits on the chip at once, the plain loop with half the
         // workgroups is faster (measured at 128 heads of 64 columns: 1.71 ms pipelined, 1.10 ms plain; at 32 heads
         // 0.81 against 0.93 ms).
         if constexpr (!DELTA && !CHD) pipe = pipe && (int64_t)B * H * zp <= 512;
