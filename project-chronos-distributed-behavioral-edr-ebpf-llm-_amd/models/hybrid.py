@@ -1,10 +1,13 @@
 """Hybrid decoders: a list of layers, each with a token mixer of some kind (recurrent matrix memory, latent
 attention, windowed or chunked attention, gated delta rule, gated linear attention, state-space duality, real-gated
-linear recurrence) and an optional feed-forward (dense, gated, mixture of experts), on a float32 residual stream.
+linear recurrence, retention, two mixers side by side) and an optional feed-forward (dense, gated, mixture of
+experts), on a float32 residual stream.
 The stream's rule is a parameter of the configuration: the norm on the sublayer's OUTPUT (``out_norm``:
-x <- x + layer_norm(sublayer(x))), AFTER the sum (``post_norm``: x <- rms_norm(alpha x + sublayer(x))) or on the
-sublayer's INPUT (``pre_norm``: x <- x + sublayer(rms_norm(x))).  A range of layers may repeat, back to back, on
-shared weights (``loop``); every run has its own pages and state.
+x <- x + layer_norm(sublayer(x))), AFTER the sum (``post_norm``: x <- rms_norm(alpha x + sublayer(x))), on the
+sublayer's INPUT (``pre_norm``: x <- x + sublayer(rms_norm(x))) or on both sides (``sandwich``:
+x <- x + norm_b(sublayer(norm_a(x))), RMS norms over ``norm_groups`` equal parts of the row).  A range of layers may
+repeat, back to back, on shared weights (``loop``), or single layers may name another layer whose weights they use
+(``share``); every run has its own pages and state.
 
 This module is the design-independent part: the mixer and feed-forward kinds with their sizes and constants as
 parameters, the cache that holds pages for the attention layers and state slots for the recurrent ones, and the
@@ -70,15 +73,22 @@ class MoEFFSpec:
     top: int
     ff: int
     act: int = hops.ACT_GELU
+    shared_ff: int = 0   # > 0: a shared expert of this size (same form, no router weight) runs for every token
+    correction: bool = True   # the checkpoint holds a per-output term that steers the router's choice
     kind: str = "moe"
 
 
 @dataclass
 class WindowAttentionSpec:
     """Grouped-query softmax attention through a sliding window that also keeps each sequence's first tokens, with
-    per-head RMS norm of queries and keys, rotation of the leading ``rope_dims`` columns (long wavelengths slowed
-    down by ``rope_scaling`` = (factor, low, high, original length)), a learned softmax sink per head, an optional
-    mix of every token's values with those of the first such layer, and a sigmoid output gate per head."""
+    per-head RMS norm of queries and keys, rotation of the leading ``rope_dims`` columns (``rope_scaling``: see
+    :func:`rope_cos_sin`), a learned softmax sink per head, an optional mix of every token's values with those of the
+    first such layer, and a sigmoid output gate (one number per head, or with ``gate_wide`` one per output column).
+    ``pool`` > 0 (with a window): beside the window's tokens a query sees one key and value per block of ``pool``
+    positions that lies wholly before its window — the means of the block's cached keys and values.  ``v_from_k``:
+    there is no value projection, the values are the keys as projected (before norm and rotation).  ``v_rot``: values
+    are cached rotated by their position over all ``vdim`` columns (frequencies rope_base^(-2m/vdim), unscaled) and
+    every head's output is turned back by the query's position."""
     heads: int
     kv_heads: int
     dim: int
@@ -96,12 +106,48 @@ class WindowAttentionSpec:
     sink: bool = True        # a learned softmax sink per head
     gate: bool = True        # a sigmoid output gate per head
     bias: bool = False       # the q, k, v projections add a bias
+    pool: int = 0            # > 0: pooled blocks of this many positions stay visible before the window
+    v_from_k: bool = False   # values = the keys as projected
+    v_rot: bool = False      # values rotated by their position, outputs turned back
+    gate_wide: bool = False  # the sigmoid output gate has heads * vdim rows instead of heads
     kind: str = "window_attention"
 
     def params(self, d: int) -> int:
-        qkv = self.heads * self.dim + self.kv_heads * (self.dim + self.vdim)
-        return d * (qkv + self.heads * self.gate) + 2 * self.dim * self.qk_norm + self.heads * self.sink + 1 + \
+        qkv = self.heads * self.dim + self.kv_heads * (self.dim + (0 if self.v_from_k else self.vdim))
+        gate = self.heads * (self.vdim if self.gate_wide else 1) * self.gate
+        return d * (qkv + gate) + 2 * self.dim * self.qk_norm + self.heads * self.sink + \
+            (1 if self.v_mix and not self.v_mix_first else 0) + \
             self.heads * self.vdim * d + qkv * self.bias
+
+
+@dataclass
+class RetentionSpec:
+    """Linear attention with one fixed decay per head and no softmax or denominator: per head a dim x vdim state
+    S <- decay_h S + k v^T, o = S^T q, with q and k rotated (``rope_dims`` leading columns) and k times dim^(-1/2);
+    each head's read-out is scaled to unit RMS and multiplied by silu of a gate projection."""
+    heads: int
+    dim: int
+    vdim: int
+    decay: tuple
+    rope_base: float = 10000.0
+    rope_dims: int = 0
+    rope_scaling: Optional[tuple] = None
+    kind: str = "retention"
+
+    def params(self, d: int) -> int:
+        return d * (2 * self.heads * self.dim + 2 * self.heads * self.vdim) + self.heads * self.vdim * d
+
+
+@dataclass
+class ParallelSpec:
+    """Two mixers side by side on the same input; the result is half the sum of their outputs, each first scaled to
+    unit RMS over the model width and multiplied by a weight of its own."""
+    left: object
+    right: object
+    kind: str = "parallel"
+
+    def params(self, d: int) -> int:
+        return self.left.params(d) + self.right.params(d) + 2 * d
 
 
 @dataclass
@@ -238,7 +284,11 @@ class HybridConfig:
     max_position: int = 8192
     architecture: str = "hybrid"
     residual: str = "out_norm"     # "out_norm": x <- x + layer_norm(y);  "post_norm": x <- rms_norm(alpha x + y);
-    #                                "pre_norm": x <- x + sublayer(rms_norm(x))
+    #                                "pre_norm": x <- x + sublayer(rms_norm(x));
+    #                                "sandwich": x <- x + norm_b(sublayer(norm_a(x)))
+    norm_groups: int = 1           # sandwich: the stream's RMS norms work on this many equal parts of a row
+    embed_scale: float = 1.0       # the embedding rows are multiplied by this
+    share: Optional[list] = None   # share[i] = j: layer i runs on layer j's weights (j itself has its own)
     residual_alpha: float = 1.0
     tied_head: bool = False        # the logits come from the embedding table
     loop: Optional[tuple] = None   # (start, stop, times): layers [start, stop) run ``times`` times, back to back
@@ -253,6 +303,8 @@ class HybridConfig:
     def runs(self) -> list:
         """Layer index of every layer run, in order (the looped range repeated); pages and state are per run."""
         n = len(self.layers)
+        if self.share is not None:
+            return [int(j) for j in self.share]
         if not self.loop or self.loop[2] <= 1:
             return list(range(n))
         a, b, t = self.loop
@@ -261,7 +313,10 @@ class HybridConfig:
     def param_count(self) -> int:
         d = self.hidden_size
         n = (1 if self.tied_head else 2) * self.vocab_size * d + d
-        for l in self.layers:
+        own = set(self.runs)
+        for i, l in enumerate(self.layers):
+            if i not in own:
+                continue
             m = l.mixer
             if hasattr(m, "params"):
                 n += m.params(d)
@@ -270,14 +325,15 @@ class HybridConfig:
             else:
                 n += d * (m.heads * (m.dim + m.rot_dim) + m.kv_rank + m.rot_dim + m.heads) + m.kv_rank
                 n += m.kv_rank * m.heads * (m.dim + m.vdim) + m.heads * m.vdim * d
-            n += d
+            n += d * (2 if self.residual == "sandwich" else 1)
             if l.ff is not None:
                 f = l.ff
-                n += d + {"dense": lambda: 2 * d * f.ff, "glu": lambda: 3 * d * f.ff,
-                          "moe": lambda: f.experts * 2 * d * f.ff + (f.experts + f.identity) * (d + 1),
-                          "moe_glu": lambda: f.experts * (3 * d * f.ff + d + 1),
-                          "moe_group_glu": lambda: f.experts * (3 * d * f.ff + d) + (
-                              3 * d * f.shared_ff + d if f.shared_ff else 0)}[f.kind]()
+                n += d * (2 if self.residual == "sandwich" else 1)
+                n += {"dense": lambda: 2 * d * f.ff, "glu": lambda: 3 * d * f.ff,
+                      "moe": lambda: (f.experts * f.ff + f.shared_ff) * 2 * d + (f.experts + f.identity) * (d + f.correction),
+                      "moe_glu": lambda: f.experts * (3 * d * f.ff + d + 1),
+                      "moe_group_glu": lambda: f.experts * (3 * d * f.ff + d) + (
+                          3 * d * f.shared_ff + d if f.shared_ff else 0)}[f.kind]()
             if self.token_side:
                 n += self.token_side * (2 * d + self.vocab_size) + d
         return n
@@ -290,12 +346,14 @@ class HybridConfig:
 
 class HybridCache:
     """Per latent-attention layer run a paged latent cache [NB, BS, kv_rank + rot_dim], per windowed-attention run
-    paged keys [NB, BS, G, D] and values [NB, BS, G, Dv], all in the activation dtype (block 0 is the engine's scratch
-    block); per recurrent run float32 state rows S [NS, H, D, Dv] (the matrix-memory layers also n [NS, H, D] and
-    m [NS, H]; the gated linear recurrence keeps S [NS, width]; layers with a short convolution also its last
-    conv - 1 inputs, ``hist`` [NS, conv - 1, C] in the activation dtype), one row per engine slot plus a scratch row
-    (``scratch_slot``) for the decode rows of slots that hold no running sequence.  Tensors are keyed by the index of
-    the layer RUN: a layer inside a loop has one set per pass.
+    paged keys [NB, BS, G, D] and values [NB, BS, G, Dv] (with pooled blocks also their means, ``kp`` / ``vp``
+    [NB, ceil(BS / pool), G, .]: block e of a sequence sits in row e % EP of the sequence's page e // EP), all in the
+    activation dtype (block 0 is the engine's scratch block); per recurrent run float32 state rows S [NS, H, D, Dv]
+    (the matrix-memory layers also n [NS, H, D] and m [NS, H]; the gated linear recurrence keeps S [NS, width];
+    layers with a short convolution also its last conv - 1 inputs, ``hist`` [NS, conv - 1, C] in the activation
+    dtype), one row per engine slot plus a scratch row (``scratch_slot``) for the decode rows of slots that hold no
+    running sequence.  Tensors are keyed by the index of the layer RUN: a layer inside a loop has one set per pass;
+    the two halves of a parallel mixer are keyed (run, 0) and (run, 1).
 
     A sequence's state needs no reset: a step whose first token sits at position 0 starts from zero."""
 
@@ -303,51 +361,66 @@ class HybridCache:
         self.num_blocks, self.block_size = num_blocks, block_size
         self.slots = slots
         self.scratch_slot = slots
-        self.lat: dict[int, torch.Tensor] = {}
-        self.S: dict[int, torch.Tensor] = {}
-        self.n: dict[int, torch.Tensor] = {}
-        self.m: dict[int, torch.Tensor] = {}
-        self.kc: dict[int, torch.Tensor] = {}
-        self.vc: dict[int, torch.Tensor] = {}
-        self.hist: dict[int, torch.Tensor] = {}
+        self.lat: dict = {}
+        self.S: dict = {}
+        self.n: dict = {}
+        self.m: dict = {}
+        self.kc: dict = {}
+        self.vc: dict = {}
+        self.kp: dict = {}
+        self.vp: dict = {}
+        self.hist: dict = {}
+        self._dev, self._at = device, act_dtype
         for li, l in enumerate(cfg.layers[i] for i in cfg.runs):
-            mx = l.mixer
-            if mx.kind == "latent_attention":
-                self.lat[li] = torch.zeros(num_blocks, block_size, mx.kv_rank + mx.rot_dim, device=device,
-                                           dtype=act_dtype)
-            elif mx.kind == "mlstm":
-                f32 = dict(device=device, dtype=torch.float32)
-                self.S[li] = torch.zeros(slots + 1, mx.heads, mx.dim, mx.vdim, **f32)
-                self.n[li] = torch.zeros(slots + 1, mx.heads, mx.dim, **f32)
-                self.m[li] = torch.zeros(slots + 1, mx.heads, **f32)
-            elif mx.kind == "window_attention":
-                pg = dict(device=device, dtype=act_dtype)
-                self.kc[li] = torch.zeros(num_blocks, block_size, mx.kv_heads, mx.dim, **pg)
-                self.vc[li] = torch.zeros(num_blocks, block_size, mx.kv_heads, mx.vdim, **pg)
-            elif mx.kind in ("delta_rule", "gla"):
-                self.S[li] = torch.zeros(slots + 1, mx.heads, mx.dim, mx.vdim, device=device, dtype=torch.float32)
-                if mx.kind == "delta_rule":
-                    ch = 2 * mx.kv_heads * mx.dim + mx.heads * mx.vdim
-                    self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), ch, device=device, dtype=act_dtype)
-            elif mx.kind == "mamba2":
-                self.S[li] = torch.zeros(slots + 1, mx.heads, mx.state, mx.vdim, device=device, dtype=torch.float32)
-                self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), mx.conv_channels, device=device,
-                                            dtype=act_dtype)
-            elif mx.kind == "rglru":
-                self.S[li] = torch.zeros(slots + 1, mx.width, device=device, dtype=torch.float32)
-                self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), mx.width, device=device, dtype=act_dtype)
+            self._alloc(li, l.mixer)
+
+    def _alloc(self, li, mx) -> None:
+        num_blocks, block_size, slots, device, act_dtype = self.num_blocks, self.block_size, self.slots, self._dev, self._at
+        if mx.kind == "parallel":
+            self._alloc((li, 0), mx.left)
+            self._alloc((li, 1), mx.right)
+        elif mx.kind == "latent_attention":
+            self.lat[li] = torch.zeros(num_blocks, block_size, mx.kv_rank + mx.rot_dim, device=device, dtype=act_dtype)
+        elif mx.kind == "mlstm":
+            f32 = dict(device=device, dtype=torch.float32)
+            self.S[li] = torch.zeros(slots + 1, mx.heads, mx.dim, mx.vdim, **f32)
+            self.n[li] = torch.zeros(slots + 1, mx.heads, mx.dim, **f32)
+            self.m[li] = torch.zeros(slots + 1, mx.heads, **f32)
+        elif mx.kind == "window_attention":
+            pg = dict(device=device, dtype=act_dtype)
+            self.kc[li] = torch.zeros(num_blocks, block_size, mx.kv_heads, mx.dim, **pg)
+            self.vc[li] = torch.zeros(num_blocks, block_size, mx.kv_heads, mx.vdim, **pg)
+            if mx.pool:
+                ep = (block_size + mx.pool - 1) // mx.pool
+                self.kp[li] = torch.zeros(num_blocks, ep, mx.kv_heads, mx.dim, **pg)
+                self.vp[li] = torch.zeros(num_blocks, ep, mx.kv_heads, mx.vdim, **pg)
+        elif mx.kind in ("delta_rule", "gla", "retention"):
+            self.S[li] = torch.zeros(slots + 1, mx.heads, mx.dim, mx.vdim, device=device, dtype=torch.float32)
+            if mx.kind == "delta_rule":
+                ch = 2 * mx.kv_heads * mx.dim + mx.heads * mx.vdim
+                self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), ch, device=device, dtype=act_dtype)
+        elif mx.kind == "mamba2":
+            self.S[li] = torch.zeros(slots + 1, mx.heads, mx.state, mx.vdim, device=device, dtype=torch.float32)
+            self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), mx.conv_channels, device=device, dtype=act_dtype)
+        elif mx.kind == "rglru":
+            self.S[li] = torch.zeros(slots + 1, mx.width, device=device, dtype=torch.float32)
+            self.hist[li] = torch.zeros(slots + 1, max(0, mx.conv - 1), mx.width, device=device, dtype=act_dtype)
 
     @staticmethod
     def bytes_per_block(cfg: HybridConfig, block_size: int, act_dtype) -> int:
         eb = 4 if act_dtype == torch.float32 else 2
-        per_token = 0
-        for l in (cfg.layers[i] for i in cfg.runs):
-            m = l.mixer
+
+        def per_page(m) -> int:   # elements one page of this mixer holds
+            if m.kind == "parallel":
+                return per_page(m.left) + per_page(m.right)
             if m.kind == "latent_attention":
-                per_token += m.kv_rank + m.rot_dim
-            elif m.kind == "window_attention":
-                per_token += m.kv_heads * (m.dim + m.vdim)
-        return max(1, block_size * per_token * eb)
+                return block_size * (m.kv_rank + m.rot_dim)
+            if m.kind == "window_attention":
+                rows = block_size + ((block_size + m.pool - 1) // m.pool if m.pool else 0)
+                return rows * m.kv_heads * (m.dim + m.vdim)
+            return 0
+
+        return max(1, sum(per_page(cfg.layers[i].mixer) for i in cfg.runs) * eb)
 
     def move_slots(self, src: torch.Tensor, dst: torch.Tensor) -> None:
         """Slot compaction: the recurrent state rows follow their sequences."""
@@ -367,6 +440,8 @@ class HybridLayerWeights:
     norm2: Optional[torch.Tensor] = None
     ff: dict = field(default_factory=dict)
     side: dict = field(default_factory=dict)   # the per-layer token input: w_gate, w_proj, norm, col0
+    norm1b: Optional[torch.Tensor] = None      # sandwich stream: the norms on the sublayers' outputs
+    norm2b: Optional[torch.Tensor] = None
 
 
 @dataclass
@@ -382,10 +457,12 @@ class HybridWeights:
         for t in (self.embed, self.final_norm, self.head, self.side_embed):
             if t is not None:
                 n += t.numel() * t.element_size()
-        for l in self.layers:
-            for t in (l.norm1, l.norm2, *l.mix.values(), *l.ff.values(), *l.side.values()):
+        for l in {id(l): l for l in self.layers}.values():   # a layer that runs on another's weights counts once
+            for t in (l.norm1, l.norm2, l.norm1b, l.norm2b, *l.mix.values(), *l.ff.values(), *l.side.values()):
                 if isinstance(t, torch.Tensor):
                     n += t.numel() * t.element_size()
+                elif isinstance(t, dict):
+                    n += sum(v.numel() * v.element_size() for v in t.values() if isinstance(v, torch.Tensor))
         return n
 
 
@@ -415,24 +492,31 @@ def pack_dense(spec: DenseFFSpec, t: dict, device, act_dtype) -> dict:
 
 
 def pack_moe(spec: MoEFFSpec, t: dict, device, act_dtype) -> dict:
-    """t: router, correction, e<k>.up, e<k>.down.  Expert weights are stacked [E, ...] for the grouped kernels."""
+    """t: router, correction (zeros when the design has none), e<k>.up, e<k>.down and, with a shared expert, shared.up, shared.down.
+    Expert weights are stacked [E, ...] for the grouped kernels."""
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
-    return dict(w_router=a(t["router"]), correction=t["correction"].to(device=device, dtype=torch.float32).contiguous(),
-                w_up=a(torch.stack([t[f"e{e}.up"] for e in range(spec.experts)])),
-                w_down=a(torch.stack([t[f"e{e}.down"] for e in range(spec.experts)])))
+    corr = t["correction"] if spec.correction else torch.zeros(spec.experts + spec.identity)
+    out = dict(w_router=a(t["router"]), correction=corr.to(device=device, dtype=torch.float32).contiguous(),
+               w_up=a(torch.stack([t[f"e{e}.up"] for e in range(spec.experts)])),
+               w_down=a(torch.stack([t[f"e{e}.down"] for e in range(spec.experts)])))
+    if spec.shared_ff:
+        out.update(ws_up=a(t["shared.up"]), ws_down=a(t["shared.down"]))
+    return out
 
 
 def pack_window_attention(spec: WindowAttentionSpec, t: dict, device, act_dtype) -> dict:
-    """t: q, k, v, q.norm, k.norm, sink, g, o and, in value-mixing layers, vmix.  q | k | v become one projection;
-    the per-head gate rows are a few-row float32-output projection."""
+    """t: q, k, v, q.norm, k.norm, sink, g, o and, in value-mixing layers, vmix.  q | k | v become one projection
+    (q | k when the values are the keys; q | k | v | g with a gate per output column); per-head gate rows are a
+    few-row float32-output projection."""
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
     f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
-    out = dict(w_qkv=a(torch.cat([t["q"], t["k"], t["v"]], 0)), w_o=a(t["o"]))
+    rows = [t["q"], t["k"]] + ([] if spec.v_from_k else [t["v"]]) + ([t["g"]] if spec.gate and spec.gate_wide else [])
+    out = dict(w_qkv=a(torch.cat(rows, 0)), w_o=a(t["o"]))
     if spec.qk_norm:
         out.update(q_norm=f(t["q.norm"]), k_norm=f(t["k.norm"]))
     if spec.sink:
         out["sink"] = f(t["sink"])
-    if spec.gate:
+    if spec.gate and not spec.gate_wide:
         out["w_g"] = a(t["g"])
     if spec.bias:
         out["b_qkv"] = a(torch.cat([t["q.b"], t["k.b"], t["v.b"]], 0))
@@ -486,6 +570,24 @@ def pack_gla(spec: GLASpec, t: dict, device, act_dtype) -> dict:
                 b_a2=f(t["a2.b"]), norm=f(t["norm"].float().repeat(spec.heads)), w_o=a(t["o"]))
 
 
+def pack_retention(spec: RetentionSpec, t: dict, device, act_dtype) -> dict:
+    """t: q, k, v, g, o.  q | k | v | g are one projection; the decays are a float32 row, one number per head."""
+    a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
+    return dict(w_proj=a(torch.cat([t["q"], t["k"], t["v"], t["g"]], 0)), w_o=a(t["o"]),
+                decay=torch.tensor(list(spec.decay), dtype=torch.float64).to(device=device, dtype=torch.float32),
+                ones=torch.ones(spec.heads * spec.vdim, device=device, dtype=torch.float32))
+
+
+def pack_parallel(spec: ParallelSpec, t: dict, device, act_dtype) -> dict:
+    """t: left.* and right.* (each side's own tensors) plus left.out and right.out, the weights of the two outputs'
+    norms over the model width."""
+    f = lambda x: x.to(device=device, dtype=torch.float32).contiguous()  # noqa: E731
+    side = lambda p: {k[len(p):]: v for k, v in t.items() if k.startswith(p) and k != p + "out"}  # noqa: E731
+    return dict(left=MIXERS[spec.left.kind][1](spec.left, side("left."), device, act_dtype),
+                right=MIXERS[spec.right.kind][1](spec.right, side("right."), device, act_dtype),
+                out_l=f(t["left.out"]), out_r=f(t["right.out"]))
+
+
 def pack_glu(spec: GluFFSpec, t: dict, device, act_dtype) -> dict:
     a = lambda x: x.to(device=device, dtype=act_dtype).contiguous()  # noqa: E731
     return dict(w_gu=a(torch.cat([t["gate"], t["up"]], 0)), w_down=a(t["down"]))
@@ -518,20 +620,37 @@ def pack_moe_group_glu(spec: MoEGroupGluSpec, t: dict, device, act_dtype) -> dic
 
 def rope_cos_sin(base: float, dims: int, max_pos: int, device, scaling: Optional[tuple] = None) -> torch.Tensor:
     """[max_pos, dims] float32: cos(p f_i) for i < dims/2, then sin(p f_i), f_i = base^(-2i/dims); angles in float64
-    before the rounding to float32.  ``scaling`` = (factor, low, high, original): frequencies whose wavelength is
-    shorter than original/high stay, those longer than original/low are divided by factor, and between the two the
-    frequency is interpolated linearly in original/wavelength."""
-    inv = base ** (-torch.arange(0, dims, 2, dtype=torch.float64) / dims)
-    if scaling is not None:
-        import math
+    before the rounding to float32.  ``scaling``:
 
+    (factor, low, high, original): frequencies whose wavelength is shorter than original/high stay, those longer than
+        original/low are divided by factor, and between the two the frequency is interpolated linearly in
+        original/wavelength;
+    ("linear", factor): every frequency is divided by factor;
+    ("ramp", factor, original, fast, slow): with n(t) = dims ln(original / (2 pi t)) / (2 ln base) the pair index at
+        which ``original`` positions make t turns, lo = max(floor(n(fast)), 0), hi = min(ceil(n(slow)), dims - 1) and
+        r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1), the frequency is f_i / factor r_i + f_i (1 - r_i), and
+        cos and sin are multiplied by 0.1 ln(factor) + 1."""
+    import math
+
+    inv = base ** (-torch.arange(0, dims, 2, dtype=torch.float64) / dims)
+    mag = 1.0
+    if scaling is not None and scaling[0] == "linear":
+        inv = inv / float(scaling[1])
+    elif scaling is not None and scaling[0] == "ramp":
+        factor, orig, fast, slow = (float(v) for v in scaling[1:])
+        where = lambda t: dims * math.log(orig / (2 * math.pi * t)) / (2 * math.log(base))  # noqa: E731
+        lo, hi = max(math.floor(where(fast)), 0), min(math.ceil(where(slow)), dims - 1)
+        r = ((torch.arange(dims // 2, dtype=torch.float64) - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        inv = inv / factor * r + inv * (1 - r)
+        mag = 0.1 * math.log(factor) + 1.0
+    elif scaling is not None:
         factor, low, high, orig = (float(v) for v in scaling)
         wl = 2 * math.pi / inv
         s = ((orig / wl - low) / (high - low)).clamp(0.0, 1.0) if high != low else torch.ones_like(inv)
         mid = (1 - s) * inv / factor + s * inv
         inv = torch.where(wl < orig / high, inv, torch.where(wl > orig / low, inv / factor, mid))
     fr = torch.outer(torch.arange(max_pos, dtype=torch.float64), inv)
-    return torch.cat([fr.cos(), fr.sin()], 1).float().to(device)
+    return (torch.cat([fr.cos(), fr.sin()], 1) * mag).float().to(device)
 
 
 # -----------------------------------------------------------------------------------------------------------------
@@ -585,20 +704,52 @@ def mix_latent_attention(model, li: int, spec: LatentAttentionSpec, w: dict, h, 
     return hops.matmul(ov, w["w_o"])
 
 
-def mix_window_attention(model, li: int, spec: WindowAttentionSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+def mix_window_attention(model, li, spec: WindowAttentionSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
     H, G, D, Dv = spec.heads, spec.kv_heads, spec.dim, spec.vdim
     qkv = hops.matmul(h, w["w_qkv"], w.get("b_qkv"))
-    gate = hops.rowdot(h, w["w_g"]) if spec.gate else None
+    gate = hops.rowdot(h, w["w_g"]) if spec.gate and not spec.gate_wide else None
     mixes = spec.v_mix and not spec.v_mix_first
+    v_tab = model.rope_v.get(li)
     v = hops.window_prep(qkv, H, G, D, Dv, meta.shared["v_first"] if mixes else None, w.get("vmix"), meta.pos,
                          meta.tok_seq, meta.block_table, w.get("q_norm"), w.get("k_norm"), model.cfg.norm_eps,
-                         model.rope.get(li), spec.rope_dims, cache.kc[li], cache.vc[li], spec.v_mix_first)
+                         model.rope.get(li), spec.rope_dims, cache.kc[li], cache.vc[li], spec.v_mix_first,
+                         H * D if spec.v_from_k else -1, v_tab)
     if spec.v_mix_first:
         meta.shared["v_first"] = v
+    pooled = spec.pool > 0 and spec.window > 0
+    if pooled:   # the blocks this step's tokens complete get their means before any query of the step looks
+        hops.pool_blocks(cache.kc[li], cache.vc[li], cache.kp[li], cache.vp[li], meta.block_table, meta.q_start,
+                         meta.pos0, spec.pool, meta.max_q)
     o = hops.window_attention(qkv, cache.kc[li], cache.vc[li], meta.block_table, meta.q_start, meta.pos, w.get("sink"),
                               gate, spec.scale, spec.window, spec.keep_first, H, model.act_dtype, meta.max_q,
-                              spec.chunk)
+                              spec.chunk, spec.pool if pooled else 0, cache.kp.get(li), cache.vp.get(li), v_tab,
+                              (H + G) * D + G * Dv if spec.gate and spec.gate_wide else -1)
     return hops.matmul(o, w["w_o"])
+
+
+def mix_retention(model, li, spec: RetentionSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    H, D, Dv = spec.heads, spec.dim, spec.vdim
+    proj = hops.matmul(h, w["w_proj"])          # q | k | v | g
+    hops.rotate_qk(proj, 0, H * D, H, H, D, spec.rope_dims, model.rope.get(li), meta.pos, 1.0, D ** -0.5)
+    o = hops.linear_scan(proj, 0, H * D, 2 * H * D, None, None, 1.0, w["decay"], None, meta.q_start, meta.pos0,
+                         meta.slots, cache.S[li], H, H, D, Dv)
+    return hops.matmul(hops.head_norm_gate(o, proj, 2 * H * D + H * Dv, w["ones"], model.cfg.norm_eps, True,
+                                           model.act_dtype), w["w_o"])
+
+
+@dataclass
+class PairOut:
+    """What a parallel mixer hands to the stream's join: the two outputs and the weights of their norms."""
+    y: torch.Tensor
+    y2: torch.Tensor
+    w: torch.Tensor
+    w2: torch.Tensor
+
+
+def mix_parallel(model, li, spec: ParallelSpec, w: dict, h, meta: StepMeta, cache: HybridCache):
+    yl = MIXERS[spec.left.kind][0](model, (li, 0), spec.left, w["left"], h, meta, cache)
+    yr = MIXERS[spec.right.kind][0](model, (li, 1), spec.right, w["right"], h, meta, cache)
+    return PairOut(yl, yr, w["out_l"], w["out_r"])
 
 
 def mix_mamba2(model, li: int, spec: Mamba2Spec, w: dict, h, meta: StepMeta, cache: HybridCache):
@@ -680,17 +831,31 @@ def ff_dense(model, spec: DenseFFSpec, w: dict, h):
 
 
 def ff_moe(model, spec: MoEFFSpec, w: dict, h):
+    """Returns the routed experts' sum and, with a shared expert, (sum, shared output): the stream's join adds both."""
     idx, wt = hops.moe_route(h, w["w_router"], w["correction"], spec.top)
-    return hops.moe_ffn(h, idx, wt, w["w_up"], w["w_down"], spec.act, model.act_dtype)
+    y = hops.moe_ffn(h, idx, wt, w["w_up"], w["w_down"], spec.act, model.act_dtype)
+    if not spec.shared_ff:
+        return y
+    return y, hops.matmul(hops.act_inplace(hops.matmul(h, w["ws_up"]), spec.act), w["ws_down"])
 
 
 MIXERS = {"mlstm": (mix_mlstm, pack_mlstm), "latent_attention": (mix_latent_attention, pack_latent),
           "window_attention": (mix_window_attention, pack_window_attention),
           "delta_rule": (mix_delta_rule, pack_delta_rule), "gla": (mix_gla, pack_gla),
-          "mamba2": (mix_mamba2, pack_mamba2), "rglru": (mix_rglru, pack_rglru)}
+          "mamba2": (mix_mamba2, pack_mamba2), "rglru": (mix_rglru, pack_rglru),
+          "retention": (mix_retention, pack_retention), "parallel": (mix_parallel, pack_parallel)}
 FEED_FORWARDS = {"dense": (ff_dense, pack_dense), "moe": (ff_moe, pack_moe), "glu": (ff_glu, pack_glu),
                  "moe_glu": (ff_moe_glu, pack_moe_glu), "moe_group_glu": (ff_moe_group_glu, pack_moe_group_glu)}
-RECURRENT_MIXERS = ("mlstm", "delta_rule", "gla", "mamba2", "rglru")
+RECURRENT_MIXERS = ("mlstm", "delta_rule", "gla", "mamba2", "rglru", "retention")
+
+
+def _is_recurrent(mx) -> bool:
+    """Does a sequence hold something beyond the tokens of its own pages?  A recurrent state; or pooled blocks, whose
+    pair sits in the page e // EP while its tokens may lie on later pages (blocks off the page grid), so that a page
+    shared between sequences as a common prefix could be written with one sequence's continuation."""
+    if mx.kind == "parallel":
+        return _is_recurrent(mx.left) or _is_recurrent(mx.right)
+    return mx.kind in RECURRENT_MIXERS or (mx.kind == "window_attention" and mx.pool > 0 and mx.window > 0)
 
 
 # -----------------------------------------------------------------------------------------------------------------
@@ -717,12 +882,29 @@ class HybridDecoder:
         self.sequence_parallel = False
         self.decode_overlap_rows = 0
         P = max_position or cfg.max_position
-        self.rope = {ri: rope_cos_sin(l.mixer.rope_base, l.mixer.rope_dims, P, self.device,
-                                      getattr(l.mixer, "rope_scaling", None))
-                     for ri, l in enumerate(cfg.layers[i] for i in cfg.runs)
-                     if l.mixer.kind in ("latent_attention", "window_attention") and l.mixer.rope_dims}
-        self.recurrent = any(l.mixer.kind in RECURRENT_MIXERS for l in cfg.layers)
-        if cfg.residual not in ("out_norm", "post_norm", "pre_norm"):
+        # rotation tables by run (the halves of a parallel mixer: (run, 0) and (run, 1)); equal tables are one tensor
+        self.rope, self.rope_v, made = {}, {}, {}
+
+        def table(base, dims, scaling):
+            key = (float(base), int(dims), tuple(scaling) if scaling else None)
+            if key not in made:
+                made[key] = rope_cos_sin(base, dims, P, self.device, scaling)
+            return made[key]
+
+        def tables(key, mx):
+            if mx.kind == "parallel":
+                tables((key, 0), mx.left)
+                tables((key, 1), mx.right)
+            elif mx.kind in ("latent_attention", "window_attention", "retention"):
+                if mx.rope_dims:
+                    self.rope[key] = table(mx.rope_base, mx.rope_dims, getattr(mx, "rope_scaling", None))
+                if getattr(mx, "v_rot", False):
+                    self.rope_v[key] = table(mx.rope_base, mx.vdim, None)
+
+        for ri, l in enumerate(cfg.layers[i] for i in cfg.runs):
+            tables(ri, l.mixer)
+        self.recurrent = any(_is_recurrent(l.mixer) for l in cfg.layers)
+        if cfg.residual not in ("out_norm", "post_norm", "pre_norm", "sandwich"):
             raise ValueError(f"unknown residual rule {cfg.residual!r}")
         if cfg.token_side and cfg.residual != "pre_norm":
             raise ValueError("the per-layer token input is part of the pre-norm stream's join")
@@ -785,9 +967,11 @@ class HybridDecoder:
         followed by decode rows)."""
         cfg, w, at = self.cfg, self.w, self.act_dtype
         meta = self._meta(sb)
-        x, h = hops.embed_rows(meta.ids, w.embed, at)
+        x, h = hops.embed_rows(meta.ids, w.embed, at, cfg.embed_scale, cfg.residual not in ("pre_norm", "sandwich"))
         if cfg.residual == "pre_norm":
             self._forward_pre_norm(x, meta, cache)
+        elif cfg.residual == "sandwich":
+            self._forward_sandwich(x, meta, cache)
         else:
             for ri, li in enumerate(cfg.runs):   # the cache is keyed by run, the weights by layer
                 spec, lw = cfg.layers[li], w.layers[li]
@@ -799,8 +983,11 @@ class HybridDecoder:
                 if self.layer_tap is not None:
                     self.layer_tap(ri, x)
         xs = x.index_select(0, meta.last_idx)
-        final = hops.layer_norm if cfg.residual == "out_norm" else hops.rms_norm
-        logits = hops.matmul(final(xs, w.final_norm, cfg.norm_eps, at), w.head).float()
+        if cfg.residual == "out_norm":
+            xn = hops.layer_norm(xs, w.final_norm, cfg.norm_eps, at)
+        else:
+            xn = hops.rms_norm(xs, w.final_norm, cfg.norm_eps, at, cfg.norm_groups if cfg.residual == "sandwich" else 1)
+        logits = hops.matmul(xn, w.head).float()
         if cfg.logit_scale != 1.0:
             logits = logits * cfg.logit_scale
         return logits if logits.dtype == logits_dtype else logits.to(logits_dtype)
@@ -834,12 +1021,39 @@ class HybridDecoder:
             if self.layer_tap is not None:
                 self.layer_tap(ri, x)
 
+    def _forward_sandwich(self, x, meta: StepMeta, cache: HybridCache) -> None:
+        """x <- x + norm1b(mixer(norm1(x))); x <- x + norm2b(ff(norm2(x))), every norm an RMS norm over
+        ``norm_groups`` equal parts of the row.  One join kernel per sublayer: it norms the sublayer's output (a
+        parallel mixer's two outputs are normed over the width and averaged first, a shared expert's output is added
+        first), adds it to the float32 stream in place and emits the norm the next sublayer reads."""
+        cfg, w, at, eps, ng = self.cfg, self.w, self.act_dtype, self.cfg.norm_eps, self.cfg.norm_groups
+        runs = cfg.runs
+        h = hops.rms_norm(x, w.layers[runs[0]].norm1, eps, at, ng) if runs else None
+        for ri, li in enumerate(runs):
+            spec, lw = cfg.layers[li], w.layers[li]
+            last = ri + 1 == len(runs)    # the last run emits nothing: the final norm reads the wanted rows only
+            nxt = None if last else w.layers[runs[ri + 1]].norm1
+            y = MIXERS[spec.mixer.kind][0](self, ri, spec.mixer, lw.mix, h, meta, cache)
+            y2 = pair = None
+            if isinstance(y, PairOut):
+                y, y2, pair = y.y, y.y2, (y.w, y.w2)
+            if spec.ff is None:
+                h = hops.sandwich_join(y, x, lw.norm1b, nxt, ng, eps, at, y2, pair, emit=not last)
+            else:
+                h = hops.sandwich_join(y, x, lw.norm1b, lw.norm2, ng, eps, at, y2, pair)
+                y = FEED_FORWARDS[spec.ff.kind][0](self, spec.ff, lw.ff, h)
+                y, y2 = y if isinstance(y, tuple) else (y, None)
+                h = hops.sandwich_join(y, x, lw.norm2b, nxt, ng, eps, at, y2, None, emit=not last)
+            if self.layer_tap is not None:
+                self.layer_tap(ri, x)
+
     def _join(self, y, x, w):
         """The residual rule: folds the sublayer output y into the float32 stream x (in place) and returns the
         stream in the activation dtype for the next sublayer."""
         cfg = self.cfg
-        if isinstance(y, tuple):
-            raise NotImplementedError("a feed-forward with a separately gated part needs the pre-norm stream")
+        if isinstance(y, (tuple, PairOut)):
+            raise NotImplementedError("a feed-forward with a separate part needs the pre-norm or the sandwich stream, "
+                                      "a parallel mixer the sandwich stream")
         if cfg.residual == "post_norm":
             return hops.scale_add_rms_norm(y, x, w, cfg.residual_alpha, cfg.norm_eps, self.act_dtype)
         return hops.add_layer_norm(y, x, w, cfg.norm_eps, self.act_dtype)

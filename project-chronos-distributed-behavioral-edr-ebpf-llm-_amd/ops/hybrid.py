@@ -60,12 +60,12 @@ def matmul(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None) -
     return torch.matmul(x, w.t())
 
 
-def embed_rows(ids, table, act_dtype):
-    """(float32 residual rows, the same rows in the activation dtype)."""
+def embed_rows(ids, table, act_dtype, scale: float = 1.0, emit: bool = True):
+    """(float32 residual rows times ``scale``, the same rows in the activation dtype or None when ``emit`` is off)."""
     if _gpu(table):
-        x = _k().hy_embed(ids, table)
-        return x, (x if _f32(act_dtype) else _k().hy_cast_bf16(x))
-    return ref.embed_rows(ids, table, act_dtype)
+        x = _k().hy_embed(ids, table, scale)
+        return x, ((x if _f32(act_dtype) else _k().hy_cast_bf16(x)) if emit else None)
+    return ref.embed_rows(ids, table, act_dtype, scale, emit)
 
 
 def layer_norm(x, w, eps: float, act_dtype):
@@ -138,10 +138,13 @@ def moe_ffn(h, idx, wt, w_up, w_down, act: int, act_dtype):
 # ---- post-norm residual stream, clamped GLU, windowed attention with sinks, linear-state recurrences ---------------
 
 
-def rms_norm(x, w, eps: float, act_dtype):
+def rms_norm(x, w, eps: float, act_dtype, groups: int = 1):
+    """``groups`` > 1: every one of that many equal parts of a row is divided by its own root mean square."""
     if _gpu(x):
+        if groups > 1:
+            return _k().hy_sandwich_join(None, None, x, None, w, None, None, groups, eps, _f32(act_dtype), False, True)
         return _k().hy_rms_norm(x, w, eps, _f32(act_dtype))
-    return ref.rms_norm(x, w, eps, act_dtype)
+    return ref.rms_norm(x, w, eps, act_dtype, groups)
 
 
 def scale_add_rms_norm(y, x, w, alpha: float, eps: float, act_dtype):
@@ -160,24 +163,43 @@ def glu(gu, limit: float, slope: float, shift: float, act_dtype):
 
 
 def window_prep(qkv, H: int, G: int, D: int, Dv: int, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm,
-                eps: float, cos_sin, dims: int, kc, vc, emit_v: bool):
+                eps: float, cos_sin, dims: int, kc, vc, emit_v: bool, v_off: int = -1, v_cos_sin=None):
+    """``v_off`` >= 0: the column of qkv where the values start (default: after the keys); ``v_cos_sin``: a rotation
+    table over all Dv columns that the values pass before they are cached."""
     if _gpu(qkv):
         v = _k().hy_window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin,
-                                dims, kc, vc, emit_v)
+                                dims, kc, vc, emit_v, v_off, v_cos_sin)
         return v if emit_v else None
     return ref.window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin,
-                           dims, kc, vc, emit_v)
+                           dims, kc, vc, emit_v, v_off, v_cos_sin)
+
+
+def pool_blocks(kc, vc, kp, vp, block_table, q_start, pos0, pool: int, max_q: int) -> None:
+    """Means of the keys and values of the blocks of ``pool`` positions that this step's tokens complete, into the
+    pooled caches.  ``max_q``: the most tokens any sequence brings in this step (sizes the launch grid)."""
+    if _gpu(kc):
+        _k().hy_pool_blocks(kc, vc, kp, vp, block_table, q_start, pos0, pool, max_q)
+    else:
+        ref.pool_blocks(kc, vc, kp, vp, block_table, q_start, pos0, pool)
 
 
 def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale: float, window: int, keep_first: int,
-                     H: int, act_dtype, max_q: int, chunk: int = 0):
+                     H: int, act_dtype, max_q: int, chunk: int = 0, pool: int = 0, kp=None, vp=None, v_cos_sin=None,
+                     g_off: int = -1):
     """``max_q``: the most tokens any sequence brings in this step (sizes the launch grid).  ``chunk`` > 0: keys
-    outside the query's own chunk of that many positions are hidden."""
+    outside the query's own chunk of that many positions are hidden.  ``pool`` > 0: the pooled pairs of the blocks
+    that lie wholly before a query's window join its softmax.  ``v_cos_sin`` [P, Dv]: every head's output is turned
+    back by the query's position (the values were cached rotated); ``g_off`` >= 0: the output is multiplied element by
+    element with sigmoid of qkv[:, g_off : g_off + H Dv].  The matrix-core kernel does both in its epilogue."""
     if _gpu(qkv):
         return _k().hy_window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first,
-                                        chunk, H, max_q)
-    return ref.window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H,
-                                act_dtype, chunk)
+                                        chunk, H, max_q, pool, kp if pool else None, vp if pool else None, v_cos_sin,
+                                        g_off)
+    o = ref.window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H,
+                             act_dtype, chunk, pool, kp, vp)
+    if v_cos_sin is not None or g_off >= 0:
+        o = ref.unrotate_gate(o, pos, v_cos_sin, qkv if g_off >= 0 else None, g_off, H, vc.shape[3], act_dtype)
+    return o
 
 
 def short_conv(x, w, tok_seq, q_start, pos0, slots, hist, silu: bool = True, bias=None, x_off: int = 0):
@@ -298,3 +320,31 @@ def moe_route_group(h, w_router, top: int, n_groups: int, keep: int, scale: floa
     if _gpu(h):
         return _k().hy_moe_route_group(h, w_router, top, n_groups, keep, scale)
     return ref.moe_route_group(h, w_router, top, n_groups, keep, scale)
+
+
+# ---- sandwich residual stream, rotated values, retention -----------------------------------------------------------
+
+
+def sandwich_join(y, x, w_y, w_out, groups: int, eps: float, act_dtype, y2=None, pair=None, emit: bool = True):
+    """x (float32 residual, in place) <- x + group_rms_norm(v) * w_y with v = y (+ y2), or with ``pair`` = (w_a, w_b)
+    v = (rms_norm(y) w_a + rms_norm(y2) w_b) / 2.  Returns group_rms_norm(x) * w_out in the activation dtype, or None
+    when ``emit`` is off."""
+    if _gpu(x):
+        h = _k().hy_sandwich_join(y, y2, x, w_y, w_out if emit else None, pair[0] if pair else None,
+                                  pair[1] if pair else None, groups, eps, _f32(act_dtype), True, emit)
+        return h if emit else None
+    return ref.sandwich_join(y, x, w_y, w_out, groups, eps, act_dtype, y2, pair, emit)
+
+
+def unrotate_gate(o, pos, v_cos_sin, gate_src, g_off: int, H: int, Dv: int, act_dtype):
+    if _gpu(o):
+        return _k().hy_unrotate_gate(o, pos, v_cos_sin, gate_src, g_off, H, Dv)
+    return ref.unrotate_gate(o, pos, v_cos_sin, gate_src, g_off, H, Dv, act_dtype)
+
+
+def rotate_qk(proj, q_off: int, k_off: int, HQ: int, HK: int, D: int, dims: int, cos_sin, pos, q_mul: float,
+              k_mul: float) -> None:
+    if _gpu(proj):
+        _k().hy_rotate_qk(proj, q_off, k_off, HQ, HK, D, dims if cos_sin is not None else 0, cos_sin, pos, q_mul, k_mul)
+    else:
+        ref.rotate_qk(proj, q_off, k_off, HQ, HK, D, dims, cos_sin, pos, q_mul, k_mul)

@@ -13,9 +13,11 @@ import torch
 ACT_RELU2, ACT_GELU = 0, 1
 
 
-def embed_rows(ids, table, act_dtype):
+def embed_rows(ids, table, act_dtype, scale=1.0, emit=True):
     x = table[ids.long()].float()
-    return x, (x if act_dtype == torch.float32 else x.to(act_dtype))
+    if scale != 1.0:
+        x = x * scale
+    return x, ((x if act_dtype == torch.float32 else x.to(act_dtype)) if emit else None)
 
 
 def layer_norm(x, w, eps, act_dtype):
@@ -192,8 +194,14 @@ def moe_ffn(h, idx, wt, w_up, w_down, act, act_dtype):
 ACT_GLU = 2  # gated unit: min(g, limit) * sigmoid(slope * g) * (clamp(u, +-limit) + shift)
 
 
-def rms_norm(x, w, eps, act_dtype):
+def rms_norm(x, w, eps, act_dtype, groups=1):
+    """``groups`` > 1: the row is split into that many equal consecutive parts, each divided by its own root mean
+    square; the whole row is multiplied by w."""
     xf = x.float()
+    if groups > 1:
+        xg = xf.view(*xf.shape[:-1], groups, xf.shape[-1] // groups)
+        xf = (xg * torch.rsqrt(xg.pow(2).mean(-1, keepdim=True) + eps)).view(xf.shape)
+        return (xf * w.float()).to(act_dtype)
     return (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + eps) * w.float()).to(act_dtype)
 
 
@@ -213,15 +221,19 @@ def glu(gu, limit, slope, shift, act_dtype):
 
 
 def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_norm, k_norm, eps, cos_sin, dims, kc, vc,
-                emit_v):
+                emit_v, v_off=-1, v_cos_sin=None):
     """qkv [T, H D + G D + G Dv]: per-head RMS norm (weights q_norm / k_norm [D], float32 math; both None: no
     norm) and rotation of the query and key heads, queries in place; values mixed with ``v_first`` [T, G Dv] as (1 - lam) v + lam v_first when
     given; keys and (mixed) values written to the paged caches kc [NB, BS, G, D], vc [NB, BS, G, Dv].  Returns the
-    values as read from the projection [T, G Dv] when ``emit_v`` (the source of later layers' mixing), else None."""
+    values as read from the projection [T, G Dv] when ``emit_v`` (the source of later layers' mixing), else None.
+    ``v_off`` >= 0: the values start at that column of qkv instead of after the keys (at H D they are the keys as
+    projected).  ``v_cos_sin`` [P, Dv]: the values are rotated by their position over all Dv columns before the
+    write."""
     T = qkv.shape[0]
     q = qkv[:, :H * D].view(T, H, D)
     k = qkv[:, H * D:(H + G) * D].view(T, G, D)
-    v = qkv[:, (H + G) * D:].view(T, G, Dv)
+    v0 = (H + G) * D if v_off < 0 else v_off
+    v = qkv[:, v0:v0 + G * Dv].view(T, G, Dv)
     out_v = v.reshape(T, G * Dv).clone() if emit_v else None
 
     def norm_rot(x, w):
@@ -236,6 +248,8 @@ def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_nor
     if v_first is not None:
         l = lam.float().reshape(())
         vf = (1.0 - l) * vf + l * v_first.view(T, G, Dv).float()
+    if v_cos_sin is not None:
+        vf = rotate_half_rows(vf, v_cos_sin, pos, Dv)
     bs = kc.shape[1]
     blk = block_table[tok_seq.long(), (pos // bs).long()].long()
     kc[blk, (pos % bs).long()] = kn.to(kc.dtype)
@@ -244,15 +258,35 @@ def window_prep(qkv, H, G, D, Dv, v_first, lam, pos, tok_seq, block_table, q_nor
     return out_v
 
 
+def pool_blocks(kc, vc, kp, vp, block_table, q_start, pos0, pool):
+    """Means of the cached keys and values of every block of ``pool`` positions whose last position is among this
+    step's tokens (sequence b brings positions pos0[b] .. pos0[b] + n_b - 1), in float32, written in the cache dtype
+    to kp / vp [NB, EP, G, .]: block e of a sequence sits in row e % EP of the sequence's page e // EP."""
+    bs, ep = kc.shape[1], kp.shape[1]
+    qs, p0 = q_start.tolist(), pos0.tolist()
+    for b in range(len(qs) - 1):
+        n = qs[b + 1] - qs[b]
+        if n <= 0:
+            continue
+        for e in range(p0[b] // pool, (p0[b] + n) // pool):
+            j = torch.arange(e * pool, (e + 1) * pool, device=kc.device)
+            pages = block_table[b, (j // bs).long()].long()
+            page = int(block_table[b, e // ep])
+            kp[page, e % ep] = kc[pages, (j % bs).long()].float().mean(0).to(kp.dtype)
+            vp[page, e % ep] = vc[pages, (j % bs).long()].float().mean(0).to(vp.dtype)
+
+
 def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, window, keep_first, H, act_dtype,
-                     chunk=0):
+                     chunk=0, pool=0, kp=None, vp=None):
     """Causal softmax attention over a paged cache through a sliding window that also keeps a sequence's first
     tokens: the query at position i sees key j <= i when i - j < window or j < keep_first (window 0: every j <= i).
     ``chunk`` > 0 further hides every key outside the query's own chunk of that many positions (the chunk grid
     is anchored at the sequence's first position): j is visible only when j // chunk == i // chunk.
     ``sink`` f32 [H] or None: exp(sink_h) joins the softmax denominator (no key, no value).  ``gate`` f32 [T, H] or
     None: head h's output times sigmoid(gate).  Queries are the first H D columns of qkv; query head h reads
-    key/value head h // (H / G).  Returns [T, H Dv]."""
+    key/value head h // (H / G).  ``pool`` > 0 (with a window): the query at i also sees the pooled pair of every
+    block e with e pool + pool - 1 <= i - window (kp / vp as :func:`pool_blocks` leaves them), in the same softmax.
+    Returns [T, H Dv]."""
     T = qkv.shape[0]
     G, D, Dv = kc.shape[2], kc.shape[3], vc.shape[3]
     q = qkv[:, :H * D].view(T, H, D).float()
@@ -278,9 +312,20 @@ def window_attention(qkv, kc, vc, block_table, q_start, pos, sink, gate, scale, 
         if chunk:
             hidden = hidden | (j < (p[:, None] // chunk) * chunk)
         sc = sc.masked_fill(hidden[:, None, :], float("-inf"))
+        nblocks = max(0, (int(p.max()) - window + 1) // pool) if pool and window else 0
+        if nblocks:
+            ep = kp.shape[1]
+            e = torch.arange(nblocks, device=qkv.device)
+            pg = block_table[b, (e // ep).long()].long()
+            pk = kp[pg, (e % ep).long()].float().repeat_interleave(rep, 1)
+            pv = vp[pg, (e % ep).long()].float().repeat_interleave(rep, 1)
+            psc = torch.einsum("thd,jhd->thj", q[t0:t1], pk) * scale
+            psc = psc.masked_fill(((e[None, :] + 1) * pool - 1 + window > p[:, None])[:, None, :], float("-inf"))
+            sc = torch.cat([sc, psc], -1)
+            vals = torch.cat([vals, pv], 0)
         if sink is not None:
             sc = torch.cat([sc, sink.float()[None, :, None].expand(t1 - t0, H, 1)], -1)
-        a = torch.softmax(sc, -1)[:, :, :ctx]
+        a = torch.softmax(sc, -1)[:, :, :ctx + nblocks]
         out[t0:t1] = torch.einsum("thj,jhv->thv", a, vals)
     if gate is not None:
         out = out * torch.sigmoid(gate.float())[:, :, None]
@@ -339,7 +384,8 @@ def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q
                 vscale=None):
     """Linear-state recurrence over a flattened token stream, per value head h (reading q/k head h // (H / HK)):
 
-        S <- decay * S                      decay f32 [T, H] (one per head) or [T, H, D] (one per key channel / row)
+        S <- decay * S                      decay f32 [T, H] (one per head), [T, H, D] (one per key channel / row)
+                                            or [H] (one per head, the same for every token)
         u  = v - S^T k, times beta          only when beta f32 [T, H] is given (the delta rule); else u = v
         S <- S + k u^T;   o = S^T q
 
@@ -361,7 +407,9 @@ def linear_scan(proj, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q
         v = v * vscale[:, :, None]
     rep = H // HK
     q, k = q.repeat_interleave(rep, 1), k.repeat_interleave(rep, 1)
-    dec = decay.view(T, H, -1, 1)  # [T, H, 1 | D, 1]
+    if decay.dim() == 1:           # one fixed number per head
+        decay = decay[None, :].expand(T, H)
+    dec = decay.reshape(T, H, -1, 1)  # [T, H, 1 | D, 1]
     for b in range(len(sl)):
         if qs[b + 1] <= qs[b]:
             continue
@@ -511,3 +559,47 @@ def moe_route_group(h, w_router, top, n_groups, keep, scale):
     idx = torch.sort(cand, dim=-1, descending=True, stable=True).indices[:, :top]
     val = torch.gather(s, 1, idx)
     return idx.to(torch.int32), val / (val.sum(-1, keepdim=True) + 1e-20) * scale
+
+
+# ---- sandwich residual stream, pooled windows, rotated values, retention --------------------------------------------
+
+
+def sandwich_join(y, x, w_y, w_out, groups, eps, act_dtype, y2=None, pair=None, emit=True):
+    """The sandwich stream's join.  v = y (+ y2), or with ``pair`` = (w_a, w_b): v = (rms_norm(y) w_a +
+    rms_norm(y2) w_b) / 2, both norms over the whole row.  Then v <- group_rms_norm(v) * w_y and x (float32, in
+    place) <- x + v.  Returns group_rms_norm(x) * w_out in the activation dtype (None when ``emit`` is off)."""
+    v = y.float()
+    if pair is not None:
+        v = 0.5 * (rms_norm(v, pair[0], eps, torch.float32) + rms_norm(y2.float(), pair[1], eps, torch.float32))
+    elif y2 is not None:
+        v = v + y2.float()
+    x.add_(rms_norm(v, w_y, eps, torch.float32, groups))
+    return rms_norm(x, w_out, eps, act_dtype, groups) if emit else None
+
+
+def unrotate_gate(o, pos, v_cos_sin, gate_src, g_off, H, Dv, act_dtype):
+    """o [T, H Dv]: every head's row is turned back by the token's position (the inverse of the rotation
+    :func:`window_prep` applies to values; skipped without a table), then multiplied element by element with sigmoid
+    of gate_src[:, g_off : g_off + H Dv] (skipped without a gate source)."""
+    T = o.shape[0]
+    of = o.float().view(T, H, Dv)
+    if v_cos_sin is not None:
+        half = Dv // 2
+        cs = v_cos_sin[pos.long()]
+        c, s = cs[:, None, :half], cs[:, None, half:]
+        u, v = of[..., :half], of[..., half:]
+        of = torch.cat([u * c + v * s, v * c - u * s], -1)
+    of = of.reshape(T, H * Dv)
+    if gate_src is not None:
+        of = of * torch.sigmoid(gate_src[:, g_off:g_off + H * Dv].float())
+    return of.to(act_dtype)
+
+
+def rotate_qk(proj, q_off, k_off, HQ, HK, D, dims, cos_sin, pos, q_mul, k_mul):
+    """In place on proj [T, C]: the HQ heads of D columns from q_off and the HK heads from k_off are rotated on their
+    first ``dims`` columns (skipped without a table) and multiplied by q_mul / k_mul, in float32."""
+    T = proj.shape[0]
+    for off, n, mul in ((q_off, HQ, q_mul), (k_off, HK, k_mul)):
+        x = proj[:, off:off + n * D].view(T, n, D)
+        xf = rotate_half_rows(x, cos_sin, pos, dims) if (cos_sin is not None and dims) else x.float()
+        x.copy_((xf * mul).to(x.dtype))
