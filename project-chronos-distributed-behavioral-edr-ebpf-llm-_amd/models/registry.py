@@ -169,6 +169,29 @@ def _tugovik_presets():
     return list(tugovik.PRESETS)
 
 
+def _vogerax_build(name, device, tp, seed, is_path, max_position, weight_dtype, dtype):
+    from . import vogerax
+
+    if tp.world > 1:
+        raise NotImplementedError("Vogerax runs on full-weight ranks (data-parallel replicas)")
+    if weight_dtype != "bf16":
+        raise NotImplementedError("Vogerax weights are served in the activation dtype (no fp8 projections)")
+    return vogerax.build(name, device, seed, DTYPES[dtype], max_position)
+
+
+def _vogerax_is_checkpoint(path: str) -> bool:
+    from . import vogerax
+
+    return vogerax.is_checkpoint(path)
+
+
+def _vogerax_presets():
+    from . import vogerax
+
+    return list(vogerax.PRESETS)
+
+
+register(Family("vogerax", _vogerax_presets, _vogerax_is_checkpoint, _vogerax_build, ("bf16", "fp32")))
 register(Family("tugovik", _tugovik_presets, _tugovik_is_checkpoint, _tugovik_build, ("bf16", "fp32")))
 register(Family("kalesun", _kalesun_presets, _kalesun_is_checkpoint, _kalesun_build, ("bf16", "fp32")))
 register(Family("zokunex", _zokunex_presets, _zokunex_is_checkpoint, _zokunex_build, ("bf16", "fp32")))
