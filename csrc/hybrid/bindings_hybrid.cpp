@@ -13,7 +13,7 @@
 #include <tuple>
 
 namespace chronos {
-void launch_hy_embed(const int32_t*, const void*, float*, int, int, bool, hipStream_t);
+void launch_hy_embed(const int32_t*, const void*, float*, int, int, float, bool, hipStream_t);
 void launch_hy_cast_bf16(const float*, uint16_t*, int64_t, hipStream_t);
 void launch_hy_layer_norm(const void*, bool, float*, const float*, void*, bool, int, int, float, hipStream_t);
 void launch_hy_rowdot(const void*, const void*, const float*, float*, int, int, int, bool, hipStream_t);
@@ -43,17 +43,26 @@ void launch_hy_head_norm_gate(const float*, const void*, int, int, const float*,
                               hipStream_t);
 void launch_hy_window_prep(void*, int, int, int, int, int, const void*, const float*, const int32_t*, const int32_t*,
                            const int32_t*, int, const float*, const float*, float, const float*, int, void*, void*, int,
-                           void*, int, bool, hipStream_t);
+                           void*, int, const float*, int, bool, hipStream_t);
+void launch_hy_pool_blocks(const void*, const void*, void*, void*, const int32_t*, int, const int32_t*, const int32_t*, int,
+                           int, int, int, int, int, int, bool, hipStream_t);
+void launch_hy_sandwich_join(const void*, const void*, float*, const float*, const float*, const float*, const float*,
+                             void*, int, int, int, float, bool, bool, hipStream_t);
+bool hy_sandwich_groups_ok(int, int);
+void launch_hy_rotate_qk(void*, int, int, int, int, int, int, int, const float*, const int32_t*, float, float, int, bool,
+                         hipStream_t);
+void launch_hy_unrotate_gate(const void*, const int32_t*, const float*, const void*, int, int, void*, int, int, int, bool,
+                             hipStream_t);
 int hy_window_rows_cap(int, int, int, bool);
 void launch_hy_window_attention(const void*, int, const void*, const void*, const int32_t*, int, const int32_t*,
                                 const int32_t*, const float*, const float*, void*, int, int, int, int, int, int, int, float,
-                                int, int, int, bool, int, float*, float*, int64_t, hipStream_t);
-int hy_window_nsplit(bool, int, int, int, int, int, int, int, int, int, int, int);
+                                int, int, int, bool, int, float*, float*, int64_t, int, int, const void*, const void*, const float*, int, hipStream_t);
+int hy_window_nsplit(bool, int, int, int, int, int, int, int, int, int, int, int, int);
 void launch_hy_short_conv(const void*, int, const float*, const float*, const int32_t*, const int32_t*, const int32_t*,
                           const int32_t*, void*, void*, int, int, int, int, bool, bool, hipStream_t);
 void launch_hy_delta_prep(const void*, int, const float*, const float*, float*, float*, float*, float*, int, int, int, int,
                           float, bool, hipStream_t);
-bool launch_hy_linear_scan(const void*, int, int, int, int, const float*, const float*, float, const float*, bool,
+bool launch_hy_linear_scan(const void*, int, int, int, int, const float*, const float*, float, const float*, bool, bool,
                            const float*, const int32_t*, const int32_t*, const int32_t*, float*, float*, int, int, int, int,
                            int, int, const float*, bool, hipStream_t);
 void launch_hy_moe_route_topk(const void*, const void*, const float*, float*, int32_t*, float*, int, int, int, int, bool,
@@ -92,13 +101,13 @@ void same_act(const Tensor& a, const Tensor& b, const char* what) {
 void i32(const Tensor& t, const char* what) { need(t.scalar_type() == at::kInt && t.is_contiguous() && t.is_cuda(), what); }
 void flt(const Tensor& t, const char* what) { need(t.scalar_type() == at::kFloat && t.is_contiguous() && t.is_cuda(), what); }
 
-Tensor hy_embed(const Tensor& ids, const Tensor& table) {
+Tensor hy_embed(const Tensor& ids, const Tensor& table, double scale) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(table.device());
     i32(ids, "embed: ids must be contiguous int32");
     need(is_act(table) && table.dim() == 2 && table.is_contiguous(), "embed: table [V, d] bf16 or f32");
     auto x = at::empty({ids.numel(), table.size(1)}, table.options().dtype(at::kFloat));
     chronos::launch_hy_embed(ids.data_ptr<int32_t>(), table.data_ptr(), x.data_ptr<float>(), (int)ids.numel(),
-                             (int)table.size(1), f32(table), stream());
+                             (int)table.size(1), (float)scale, f32(table), stream());
     return x;
 }
 
@@ -352,13 +361,19 @@ Tensor hy_head_norm_gate(const Tensor& o, const Tensor& src, int64_t g_off, cons
 Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, const c10::optional<Tensor>& v_first,
                       const c10::optional<Tensor>& lam, const Tensor& pos, const Tensor& tok_seq, const Tensor& block_table,
                       const c10::optional<Tensor>& q_norm, const c10::optional<Tensor>& k_norm, double eps,
-                      const c10::optional<Tensor>& cos_sin, int64_t dims, Tensor& kc, Tensor& vc, bool emit_v) {
+                      const c10::optional<Tensor>& cos_sin, int64_t dims, Tensor& kc, Tensor& vc, bool emit_v,
+                      int64_t v_off, const c10::optional<Tensor>& v_cos_sin) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
     same_act(qkv, kc, "window_prep: the caches hold the activation dtype");
     same_act(qkv, vc, "window_prep: the caches hold the activation dtype");
     need(qkv.dim() == 2 && qkv.is_contiguous() && kc.dim() == 4 && vc.dim() == 4 && kc.is_contiguous() && vc.is_contiguous(), "window_prep: layouts");
     const int64_t T = qkv.size(0);
-    need(H >= 1 && G >= 1 && H % G == 0 && D >= 1 && Dv >= 1 && qkv.size(1) == (H + G) * D + G * Dv, "window_prep: qkv width");
+    if (v_off < 0) v_off = (H + G) * D;   // the values follow the keys
+    need(H >= 1 && G >= 1 && H % G == 0 && D >= 1 && Dv >= 1 && qkv.size(1) >= (H + G) * D && v_off + G * Dv <= qkv.size(1), "window_prep: qkv width");
+    if (v_cos_sin) {
+        flt(*v_cos_sin, "window_prep: float32 cos/sin table of the values");
+        need(Dv % 2 == 0 && v_cos_sin->dim() == 2 && v_cos_sin->size(1) == Dv, "window_prep: the values' table is [P, Dv], Dv even");
+    }
     need(kc.size(2) == G && kc.size(3) == D && vc.size(2) == G && vc.size(3) == Dv && vc.size(0) == kc.size(0) && vc.size(1) == kc.size(1), "window_prep: cache shapes");
     i32(pos, "window_prep: pos"); i32(tok_seq, "window_prep: tok_seq"); i32(block_table, "window_prep: block_table");
     need(pos.numel() == T && tok_seq.numel() == T && block_table.dim() == 2, "window_prep: per-token metadata");
@@ -387,14 +402,16 @@ Tensor hy_window_prep(Tensor& qkv, int64_t H, int64_t G, int64_t D, int64_t Dv, 
                                    (int)block_table.size(1), q_norm ? q_norm->data_ptr<float>() : nullptr,
                                    k_norm ? k_norm->data_ptr<float>() : nullptr, (float)eps,
                                    dims > 0 ? cos_sin->data_ptr<float>() : nullptr, (int)dims, kc.data_ptr(), vc.data_ptr(),
-                                   (int)kc.size(1), emit_v ? v_out.data_ptr() : nullptr, (int)T, f32(qkv), stream());
+                                   (int)kc.size(1), emit_v ? v_out.data_ptr() : nullptr, (int)v_off,
+                                   v_cos_sin ? v_cos_sin->data_ptr<float>() : nullptr, (int)T, f32(qkv), stream());
     return v_out;
 }
 
 Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc, const Tensor& block_table,
                            const Tensor& q_start, const Tensor& pos, const c10::optional<Tensor>& sink,
                            const c10::optional<Tensor>& gate, double scale, int64_t window, int64_t keep, int64_t chunk,
-                           int64_t H, int64_t max_q) {
+                           int64_t H, int64_t max_q, int64_t pool, const c10::optional<Tensor>& kp,
+                           const c10::optional<Tensor>& vp, const c10::optional<Tensor>& v_cos_sin, int64_t g_off) {
     c10::hip::HIPGuardMasqueradingAsCUDA g(qkv.device());
     same_act(qkv, kc, "window_attention: queries and caches in one activation dtype");
     same_act(qkv, vc, "window_attention: queries and caches in one activation dtype");
@@ -408,11 +425,27 @@ Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc
     need(block_table.dim() == 2 && block_table.size(0) >= B && pos.numel() == T && window >= 0 && keep >= 0 && chunk >= 0, "window_attention: metadata");
     if (sink) { flt(*sink, "window_attention: float32 sinks"); need(sink->numel() == H, "window_attention: sink [H]"); }
     if (gate) { flt(*gate, "window_attention: float32 gate"); need(gate->numel() == T * H, "window_attention: gate [T, H]"); }
+    int64_t EP = 1;
+    if (pool > 0) {   // pooled pairs: block e of a sequence in row e % EP of its page e / EP
+        need(kp.has_value() && vp.has_value() && window > 0, "window_attention: pooled blocks need their caches and a window");
+        same_act(qkv, *kp, "window_attention: pooled caches in the activation dtype");
+        same_act(qkv, *vp, "window_attention: pooled caches in the activation dtype");
+        EP = (kc.size(1) + pool - 1) / pool;
+        need(kp->is_contiguous() && vp->is_contiguous() && kp->dim() == 4 && vp->dim() == 4 && kp->size(0) == kc.size(0) &&
+                 vp->size(0) == kc.size(0) && kp->size(1) == EP && vp->size(1) == EP && kp->size(2) == G && vp->size(2) == G &&
+                 kp->size(3) == D && vp->size(3) == Dv, "window_attention: pooled caches [NB, ceil(BS / pool), G, .]");
+    }
+    if (v_cos_sin) {   // the outputs are turned back by the query's position
+        flt(*v_cos_sin, "window_attention: float32 cos/sin table of the values");
+        need(Dv % 2 == 0 && v_cos_sin->dim() == 2 && v_cos_sin->size(1) == Dv, "window_attention: the values' table is [P, Dv], Dv even");
+    }
+    need(g_off < 0 || g_off + H * Dv <= qkv.size(1), "window_attention: the gate columns lie in the projection's row");
     auto out = at::empty({T, H * Dv}, qkv.options());
     if (T == 0 || B <= 0) return out;
     const int mq = (int)std::max<int64_t>(1, max_q);
     const int nsplit = chronos::hy_window_nsplit(f32(qkv), (int)qkv.size(1), (int)B, mq, (int)H, (int)G, (int)D, (int)Dv,
-                                                 (int)window, (int)keep, (int)chunk, (int)(block_table.size(1) * kc.size(1)));
+                                                 (int)window, (int)keep, (int)chunk, (int)(block_table.size(1) * kc.size(1)),
+                                                 (int)pool);
     Tensor part_o, part_ml;
     if (nsplit > 1) {
         part_o = at::empty({T * H * nsplit, Dv}, qkv.options().dtype(at::kFloat));
@@ -425,7 +458,10 @@ Tensor hy_window_attention(const Tensor& qkv, const Tensor& kc, const Tensor& vc
                                         out.data_ptr(), (int)B, mq, (int)H, (int)G, (int)D, (int)Dv, (int)kc.size(1),
                                         (float)scale, (int)window, (int)keep, (int)chunk, f32(qkv), nsplit,
                                         nsplit > 1 ? part_o.data_ptr<float>() : nullptr,
-                                        nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, T * H, stream());
+                                        nsplit > 1 ? part_ml.data_ptr<float>() : nullptr, T * H, (int)pool, (int)EP,
+                                        pool > 0 ? kp->data_ptr() : nullptr, pool > 0 ? vp->data_ptr() : nullptr,
+                                        v_cos_sin ? v_cos_sin->data_ptr<float>() : nullptr, g_off >= 0 ? (int)g_off : -1,
+                                        stream());
     return out;
 }
 
@@ -474,8 +510,9 @@ Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t 
     need(HK >= 1 && H % HK == 0 && D >= 1 && Dv >= 1, "linear_scan: head counts");
     need(q_off >= 0 && k_off >= 0 && v_off >= 0 && q_off + HK * D <= C && k_off + HK * D <= C && v_off + H * Dv <= C, "linear_scan: column ranges");
     flt(decay, "linear_scan: float32 decay");
-    const bool chd = decay.numel() == T * H * D && D > 1;
-    need(chd || decay.numel() == T * H, "linear_scan: decay [T, H] or [T, H, D]");
+    const bool fixed = decay.dim() == 1 && decay.numel() == H;   // one number per head, the same for every token
+    const bool chd = !fixed && decay.numel() == T * H * D && D > 1;
+    need(fixed || chd || decay.numel() == T * H, "linear_scan: decay [T, H], [T, H, D] or [H]");
     if (qscale) { flt(*qscale, "linear_scan: qscale"); need(qscale->numel() == T * HK, "linear_scan: qscale [T, HK]"); }
     if (kscale) { flt(*kscale, "linear_scan: kscale"); need(kscale->numel() == T * HK, "linear_scan: kscale [T, HK]"); }
     if (beta) { flt(*beta, "linear_scan: beta"); need(beta->numel() == T * H, "linear_scan: beta [T, H]"); }
@@ -488,7 +525,7 @@ Tensor hy_linear_scan(const Tensor& proj, int64_t q_off, int64_t k_off, int64_t 
     if (T == 0) return o;
     const bool ok = chronos::launch_hy_linear_scan(
         proj.data_ptr(), (int)C, (int)q_off, (int)k_off, (int)v_off, qscale ? qscale->data_ptr<float>() : nullptr,
-        kscale ? kscale->data_ptr<float>() : nullptr, (float)q_mul, decay.data_ptr<float>(), chd,
+        kscale ? kscale->data_ptr<float>() : nullptr, (float)q_mul, decay.data_ptr<float>(), chd, fixed,
         beta ? beta->data_ptr<float>() : nullptr, q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(),
         slots.data_ptr<int32_t>(), S.data_ptr<float>(), o.data_ptr<float>(), (int)T, (int)B, (int)HK, (int)H, (int)D, (int)Dv,
         vscale ? vscale->data_ptr<float>() : nullptr, f32(proj), stream());
@@ -660,10 +697,119 @@ std::tuple<Tensor, Tensor> hy_moe_route_group(const Tensor& h, const Tensor& w, 
     return {idx, wt};
 }
 
+void hy_pool_blocks(const Tensor& kc, const Tensor& vc, Tensor& kp, Tensor& vp, const Tensor& block_table,
+                    const Tensor& q_start, const Tensor& pos0, int64_t pool, int64_t max_q) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(kc.device());
+    same_act(kc, vc, "pool_blocks: caches in one activation dtype");
+    same_act(kc, kp, "pool_blocks: caches in one activation dtype");
+    same_act(kc, vp, "pool_blocks: caches in one activation dtype");
+    need(kc.dim() == 4 && vc.dim() == 4 && kp.dim() == 4 && vp.dim() == 4 && kc.is_contiguous() && vc.is_contiguous() &&
+             kp.is_contiguous() && vp.is_contiguous(), "pool_blocks: layouts");
+    const int64_t BS = kc.size(1), G = kc.size(2), D = kc.size(3), Dv = vc.size(3);
+    need(pool >= 1, "pool_blocks: pool >= 1");
+    const int64_t EP = (BS + pool - 1) / pool;
+    need(vc.size(0) == kc.size(0) && vc.size(1) == BS && vc.size(2) == G && kp.size(0) == kc.size(0) && vp.size(0) == kc.size(0) &&
+             kp.size(1) == EP && vp.size(1) == EP && kp.size(2) == G && vp.size(2) == G && kp.size(3) == D && vp.size(3) == Dv,
+         "pool_blocks: pooled caches [NB, ceil(BS / pool), G, .]");
+    i32(block_table, "pool_blocks: block_table"); i32(q_start, "pool_blocks: q_start"); i32(pos0, "pool_blocks: pos0");
+    const int64_t B = pos0.numel();
+    need(block_table.dim() == 2 && block_table.size(0) >= B && q_start.numel() == B + 1, "pool_blocks: metadata");
+    chronos::launch_hy_pool_blocks(kc.data_ptr(), vc.data_ptr(), kp.data_ptr(), vp.data_ptr(), block_table.data_ptr<int32_t>(),
+                                   (int)block_table.size(1), q_start.data_ptr<int32_t>(), pos0.data_ptr<int32_t>(), (int)pool,
+                                   (int)BS, (int)EP, (int)(G * D), (int)(G * Dv), (int)B, (int)std::max<int64_t>(1, max_q),
+                                   f32(kc), stream());
+}
+
+// add: x <- x + norm(v) w_y with v from y (and y2); else the plain grouped norm of x.  emit: returns norm(x) w_out.
+Tensor hy_sandwich_join(const c10::optional<Tensor>& y, const c10::optional<Tensor>& y2, Tensor& x,
+                        const c10::optional<Tensor>& w_y, const c10::optional<Tensor>& w_out,
+                        const c10::optional<Tensor>& w_a, const c10::optional<Tensor>& w_b, int64_t groups, double eps,
+                        bool out_f32, bool add, bool emit) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(x.device());
+    flt(x, "sandwich_join: the stream is contiguous float32");
+    need(x.dim() == 2, "sandwich_join: x [T, d]");
+    const int64_t T = x.size(0), d = x.size(1);
+    need(chronos::hy_sandwich_groups_ok((int)d, (int)groups), "sandwich_join: groups >= 1 and d % groups == 0");
+    need(add == y.has_value() && (add || emit), "sandwich_join: an addend when adding, something to do otherwise");
+    if (add) {
+        need(is_act(*y) && y->is_contiguous() && y->dim() == 2 && y->size(0) == T && y->size(1) == d, "sandwich_join: y [T, d]");
+        need(w_y.has_value(), "sandwich_join: the addend's norm weight");
+        flt(*w_y, "sandwich_join: float32 norm weight");
+        need(w_y->numel() == d, "sandwich_join: w_y [d]");
+        if (y2) {
+            same_act(*y, *y2, "sandwich_join: both addends in one dtype");
+            need(y2->is_contiguous() && y2->numel() == T * d, "sandwich_join: y2 [T, d]");
+        }
+        need(w_a.has_value() == w_b.has_value() && (!w_a || y2), "sandwich_join: the pair form takes two addends and two weights");
+        if (w_a) {
+            flt(*w_a, "sandwich_join: float32 pair weight"); flt(*w_b, "sandwich_join: float32 pair weight");
+            need(w_a->numel() == d && w_b->numel() == d, "sandwich_join: pair weights [d]");
+        }
+    }
+    Tensor h;
+    if (emit) {
+        need(w_out.has_value(), "sandwich_join: the emitted norm's weight");
+        flt(*w_out, "sandwich_join: float32 norm weight");
+        need(w_out->numel() == d, "sandwich_join: w_out [d]");
+        h = at::empty({T, d}, x.options().dtype(out_f32 ? at::kFloat : at::kBFloat16));
+    } else {
+        h = at::empty({0}, x.options());
+    }
+    chronos::launch_hy_sandwich_join(add ? y->data_ptr() : nullptr, (add && y2) ? y2->data_ptr() : nullptr, x.data_ptr<float>(),
+                                     add ? w_y->data_ptr<float>() : nullptr, emit ? w_out->data_ptr<float>() : nullptr,
+                                     (add && w_a) ? w_a->data_ptr<float>() : nullptr,
+                                     (add && w_b) ? w_b->data_ptr<float>() : nullptr, emit ? h.data_ptr() : nullptr, (int)T,
+                                     (int)d, (int)groups, (float)eps, add ? f32(*y) : true, out_f32, stream());
+    return h;
+}
+
+void hy_rotate_qk(Tensor& proj, int64_t q_off, int64_t k_off, int64_t HQ, int64_t HK, int64_t D, int64_t dims,
+                  const c10::optional<Tensor>& cos_sin, const Tensor& pos, double q_mul, double k_mul) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(proj.device());
+    need(is_act(proj) && proj.dim() == 2 && proj.is_contiguous(), "rotate_qk: proj [T, C]");
+    const int64_t T = proj.size(0), C = proj.size(1);
+    need(HQ >= 0 && HK >= 0 && D >= 1 && q_off >= 0 && k_off >= 0 && q_off + HQ * D <= C && k_off + HK * D <= C, "rotate_qk: column ranges");
+    need(dims >= 0 && dims % 2 == 0 && dims <= D, "rotate_qk: rotated columns");
+    if (dims > 0) {
+        need(cos_sin.has_value(), "rotate_qk: rotation needs the cos/sin table");
+        flt(*cos_sin, "rotate_qk: float32 cos/sin table");
+        need(cos_sin->dim() == 2 && cos_sin->size(1) == dims, "rotate_qk: table width");
+    }
+    i32(pos, "rotate_qk: pos");
+    need(pos.numel() == T, "rotate_qk: pos [T]");
+    chronos::launch_hy_rotate_qk(proj.data_ptr(), (int)C, (int)q_off, (int)k_off, (int)HQ, (int)HK, (int)D, (int)dims,
+                                 dims > 0 ? cos_sin->data_ptr<float>() : nullptr, pos.data_ptr<int32_t>(), (float)q_mul,
+                                 (float)k_mul, (int)T, f32(proj), stream());
+}
+
+Tensor hy_unrotate_gate(const Tensor& o, const Tensor& pos, const c10::optional<Tensor>& cos_sin,
+                        const c10::optional<Tensor>& gate_src, int64_t g_off, int64_t H, int64_t Dv) {
+    c10::hip::HIPGuardMasqueradingAsCUDA g(o.device());
+    need(is_act(o) && o.dim() == 2 && o.is_contiguous() && o.size(1) == H * Dv, "unrotate_gate: o [T, H Dv]");
+    const int64_t T = o.size(0);
+    need(cos_sin.has_value() || gate_src.has_value(), "unrotate_gate: a table or a gate");
+    if (cos_sin) {
+        flt(*cos_sin, "unrotate_gate: float32 cos/sin table");
+        need(Dv % 2 == 0 && cos_sin->dim() == 2 && cos_sin->size(1) == Dv, "unrotate_gate: table [P, Dv], Dv even");
+    }
+    if (gate_src) {
+        same_act(o, *gate_src, "unrotate_gate: the gate's source in the activation dtype");
+        need(gate_src->dim() == 2 && gate_src->is_contiguous() && gate_src->size(0) == T && g_off >= 0 &&
+                 g_off + H * Dv <= gate_src->size(1), "unrotate_gate: gate columns");
+    }
+    i32(pos, "unrotate_gate: pos");
+    need(pos.numel() == T, "unrotate_gate: pos [T]");
+    auto out = at::empty_like(o);
+    chronos::launch_hy_unrotate_gate(o.data_ptr(), pos.data_ptr<int32_t>(), cos_sin ? cos_sin->data_ptr<float>() : nullptr,
+                                     gate_src ? gate_src->data_ptr() : nullptr, gate_src ? (int)gate_src->size(1) : 0,
+                                     (int)g_off, out.data_ptr(), (int)T, (int)H, (int)Dv, f32(o), stream());
+    return out;
+}
+
 }  // namespace
 
 TORCH_LIBRARY_FRAGMENT(chronos, m) {
-    m.def("hy_embed(Tensor ids, Tensor table) -> Tensor");
+    m.def("hy_embed(Tensor ids, Tensor table, float scale=1.0) -> Tensor");
     m.def("hy_cast_bf16(Tensor x) -> Tensor");
     m.def("hy_layer_norm(Tensor x, Tensor w, float eps, bool out_f32) -> Tensor");
     m.def("hy_add_layer_norm(Tensor y, Tensor(a!) x, Tensor w, float eps, bool out_f32) -> Tensor");
@@ -685,9 +831,17 @@ TORCH_LIBRARY_FRAGMENT(chronos, m) {
     m.def("hy_head_norm_gate(Tensor o, Tensor src, int g_off, Tensor w, float eps, bool silu_gate, bool out_f32) -> Tensor");
     m.def("hy_window_prep(Tensor(a!) qkv, int H, int G, int D, int Dv, Tensor? v_first, Tensor? lam, Tensor pos, "
           "Tensor tok_seq, Tensor block_table, Tensor? q_norm, Tensor? k_norm, float eps, Tensor? cos_sin, int dims, "
-          "Tensor(b!) kc, Tensor(c!) vc, bool emit_v) -> Tensor");
+          "Tensor(b!) kc, Tensor(c!) vc, bool emit_v, int v_off=-1, Tensor? v_cos_sin=None) -> Tensor");
     m.def("hy_window_attention(Tensor qkv, Tensor kc, Tensor vc, Tensor block_table, Tensor q_start, Tensor pos, "
-          "Tensor? sink, Tensor? gate, float scale, int window, int keep, int chunk, int H, int max_q) -> Tensor");
+          "Tensor? sink, Tensor? gate, float scale, int window, int keep, int chunk, int H, int max_q, int pool=0, "
+          "Tensor? kp=None, Tensor? vp=None, Tensor? v_cos_sin=None, int g_off=-1) -> Tensor");
+    m.def("hy_pool_blocks(Tensor kc, Tensor vc, Tensor(a!) kp, Tensor(b!) vp, Tensor block_table, Tensor q_start, "
+          "Tensor pos0, int pool, int max_q) -> ()");
+    m.def("hy_sandwich_join(Tensor? y, Tensor? y2, Tensor(a!) x, Tensor? w_y, Tensor? w_out, Tensor? w_a, Tensor? w_b, "
+          "int groups, float eps, bool out_f32, bool add, bool emit) -> Tensor");
+    m.def("hy_rotate_qk(Tensor(a!) proj, int q_off, int k_off, int HQ, int HK, int D, int dims, Tensor? cos_sin, Tensor pos, "
+          "float q_mul, float k_mul) -> ()");
+    m.def("hy_unrotate_gate(Tensor o, Tensor pos, Tensor? cos_sin, Tensor? gate_src, int g_off, int H, int Dv) -> Tensor");
     m.def("hy_short_conv(Tensor x, Tensor w, Tensor tok_seq, Tensor q_start, Tensor pos0, Tensor slots, Tensor(a!) hist, "
           "bool silu, Tensor? bias, int x_off) -> Tensor");
     m.def("hy_delta_prep(Tensor y, Tensor ab, Tensor a_log, int HK, int H, int D, float q_mul) -> (Tensor, Tensor, Tensor, Tensor)");
@@ -728,6 +882,10 @@ TORCH_LIBRARY_IMPL(chronos, CUDA, m) {
     m.impl("hy_head_norm_gate", &hy_head_norm_gate);
     m.impl("hy_window_prep", &hy_window_prep);
     m.impl("hy_window_attention", &hy_window_attention);
+    m.impl("hy_pool_blocks", &hy_pool_blocks);
+    m.impl("hy_sandwich_join", &hy_sandwich_join);
+    m.impl("hy_rotate_qk", &hy_rotate_qk);
+    m.impl("hy_unrotate_gate", &hy_unrotate_gate);
     m.impl("hy_short_conv", &hy_short_conv);
     m.impl("hy_delta_prep", &hy_delta_prep);
     m.impl("hy_linear_scan", &hy_linear_scan);

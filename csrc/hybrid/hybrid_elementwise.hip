@@ -11,10 +11,10 @@ namespace hy {
 
 template <typename T>
 __global__ void __launch_bounds__(256) embed_kernel(const int32_t* __restrict__ ids, const T* __restrict__ table,
-                                                    float* __restrict__ x, int d) {
+                                                    float* __restrict__ x, int d, float scale) {
     const int64_t t = blockIdx.x;
     const T* src = table + (int64_t)ids[t] * d;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) x[t * d + i] = ld<T>(src + i);
+    for (int i = threadIdx.x; i < d; i += blockDim.x) x[t * d + i] = ld<T>(src + i) * scale;
 }
 
 __global__ void __launch_bounds__(256) cast_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ y, int64_t n) {
@@ -134,10 +134,10 @@ __global__ void __launch_bounds__(256) act_kernel(T* __restrict__ x, int64_t n, 
 
 }  // namespace hy
 
-void launch_hy_embed(const int32_t* ids, const void* table, float* x, int T, int d, bool f32, hipStream_t s) {
+void launch_hy_embed(const int32_t* ids, const void* table, float* x, int T, int d, float scale, bool f32, hipStream_t s) {
     if (T == 0) return;
-    if (f32) hy::embed_kernel<float><<<T, 256, 0, s>>>(ids, (const float*)table, x, d);
-    else hy::embed_kernel<uint16_t><<<T, 256, 0, s>>>(ids, (const uint16_t*)table, x, d);
+    if (f32) hy::embed_kernel<float><<<T, 256, 0, s>>>(ids, (const float*)table, x, d, scale);
+    else hy::embed_kernel<uint16_t><<<T, 256, 0, s>>>(ids, (const uint16_t*)table, x, d, scale);
 }
 void launch_hy_cast_bf16(const float* x, uint16_t* y, int64_t n, hipStream_t s) {
     if (n == 0) return;

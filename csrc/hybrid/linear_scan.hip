@@ -123,7 +123,7 @@ template <> __device__ __forceinline__ uint16_t zero_of<uint16_t>() { return 0; 
 template <typename T, int DP, bool DELTA, bool CHD, bool PIPE>
 __global__ void __launch_bounds__(256) linear_scan_kernel(
         const T* __restrict__ proj, int ldp, int q_off, int k_off, int v_off, const float* __restrict__ qscale,
-        const float* __restrict__ kscale, float q_mul, const float* __restrict__ decay, const float* __restrict__ beta,
+        const float* __restrict__ kscale, float q_mul, const float* __restrict__ decay, int dts, const float* __restrict__ beta,
         const int32_t* __restrict__ q_start, const int32_t* __restrict__ pos0, const int32_t* __restrict__ slots,
         float* __restrict__ S, float* __restrict__ o, int HK, int H, int D, int Dv, const float* __restrict__ vscale) {
     constexpr int TC = kScanTC, RG = PIPE ? kScanRGPrefill : kScanRGDecode, CW = 64 / RG, RL = DP / RG;
@@ -173,7 +173,7 @@ __global__ void __launch_bounds__(256) linear_scan_kernel(
         if (threadIdx.x < TC) {
             const bool ok = (int)threadIdx.x < nt;
             const int64_t t = tb + threadIdx.x;
-            sraw[0] = (!CHD && ok) ? decay[t * H + hd] : 1.f;
+            sraw[0] = (!CHD && ok) ? decay[t * dts + hd] : 1.f;   // dts = 0: the same decays for every token
             sraw[1] = (DELTA && ok) ? beta[t * H + hd] : 0.f;
             sraw[2] = (qscale != nullptr && ok) ? qscale[t * HK + hk] : q_mul;
             sraw[3] = (kscale != nullptr && ok) ? kscale[t * HK + hk] : 1.f;
@@ -381,7 +381,7 @@ void launch_hy_delta_prep(const void* y, int ldy, const float* ab, const float* 
 
 template <typename T, int DP, bool DELTA, bool CHD>
 static void linear_scan_launch(bool pipe, const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
-                               const float* kscale, float q_mul, const float* decay, const float* beta,
+                               const float* kscale, float q_mul, const float* decay, int dts, const float* beta,
                                const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int B,
                                int HK, int H, int D, int Dv, const float* vscale, hipStream_t s) {
     constexpr bool HAS_PIPE = !(DELTA && CHD);   // the combinations with a pipelined token loop
@@ -394,23 +394,23 @@ static void linear_scan_launch(bool pipe, const T* proj, int ldp, int q_off, int
         if constexpr (!DELTA && !CHD) pipe = pipe && (int64_t)B * H * zp <= 512;
         if (pipe) {
             const dim3 grid(B, H, zp);
-            hy::linear_scan_kernel<T, DP, DELTA, CHD, true><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
+            hy::linear_scan_kernel<T, DP, DELTA, CHD, true><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, dts,
                                                                                 beta, q_start, pos0, slots, S, o, HK, H, D, Dv, vscale);
             return;
         }
     }
     const dim3 grid(B, H, (Dv + 4 * (64 / hy::kScanRGDecode) - 1) / (4 * (64 / hy::kScanRGDecode)));
-    hy::linear_scan_kernel<T, DP, DELTA, CHD, false><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay,
+    hy::linear_scan_kernel<T, DP, DELTA, CHD, false><<<grid, 256, 0, s>>>(proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, dts,
                                                                          beta, q_start, pos0, slots, S, o, HK, H, D, Dv, vscale);
 }
 
 template <typename T, bool DELTA, bool CHD>
 static bool linear_scan_d(bool pipe, const T* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
-                          const float* kscale, float q_mul, const float* decay, const float* beta, const int32_t* q_start,
+                          const float* kscale, float q_mul, const float* decay, int dts, const float* beta, const int32_t* q_start,
                           const int32_t* pos0, const int32_t* slots, float* S, float* o, int B, int HK, int H, int D,
                           int Dv, const float* vscale, hipStream_t s) {
 #define HY_LS(DP)                                                                                                     \
-    linear_scan_launch<T, DP, DELTA, CHD>(pipe, proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, q_start, \
+    linear_scan_launch<T, DP, DELTA, CHD>(pipe, proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, dts, beta, q_start, \
                                           pos0, slots, S, o, B, HK, H, D, Dv, vscale, s)
     if (D <= 32) HY_LS(32);
     else if (D <= 64) HY_LS(64);
@@ -423,16 +423,18 @@ static bool linear_scan_d(bool pipe, const T* proj, int ldp, int q_off, int k_of
 
 // delta: beta != nullptr.  vscale (float [T, H], may be nullptr; without delta only): a factor on the written value.
 // chd: decay holds one number per state row ([T, H, D]) instead of one per head ([T, H]).
+// fixed (not with chd): decay holds one number per head for all tokens ([H]).
 // Returns false when D has no instantiation (D > 256).
 bool launch_hy_linear_scan(const void* proj, int ldp, int q_off, int k_off, int v_off, const float* qscale,
-                           const float* kscale, float q_mul, const float* decay, bool chd, const float* beta,
+                           const float* kscale, float q_mul, const float* decay, bool chd, bool fixed, const float* beta,
                            const int32_t* q_start, const int32_t* pos0, const int32_t* slots, float* S, float* o, int T,
                            int B, int HK, int H, int D, int Dv, const float* vscale, bool f32, hipStream_t s) {
     if (B == 0) return true;
     const bool pipe = T > B;   // some sequence brings more than one token
     const bool delta = beta != nullptr;
+    const int dts = fixed ? 0 : H;
 #define HY_LSD(T, DELTA, CHD)                                                                                        \
-    return linear_scan_d<T, DELTA, CHD>(pipe, (const T*)proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, beta, \
+    return linear_scan_d<T, DELTA, CHD>(pipe, (const T*)proj, ldp, q_off, k_off, v_off, qscale, kscale, q_mul, decay, dts, beta, \
                                         q_start, pos0, slots, S, o, B, HK, H, D, Dv, vscale, s)
     if (f32) {
         if (delta && chd) HY_LSD(float, true, true);
