@@ -87,9 +87,9 @@ def parse():
     ap.add_argument("--design-compare", action="store_true",
                     help="instead of the headline: prefill / decode throughput of the Zokunex hybrid design beside "
                          "Llama at equal width and depth, and its kernels beside their Llama counterparts")
-    ap.add_argument("--design", default="zokunex", choices=["zokunex", "kalesun", "tugovik"],
+    ap.add_argument("--design", default="zokunex", choices=["zokunex", "kalesun", "tugovik", "vogerax"],
                     help="with --design-compare: the hybrid design to measure (kalesun stands beside zokunex and llama, "
-                         "tugovik beside kalesun and llama)")
+                         "tugovik and vogerax beside kalesun and llama)")
     ap.add_argument("--design-sizes", default="1k,2k,4k", help="with --design-compare: widths to measure")
     return ap.parse_args()
 

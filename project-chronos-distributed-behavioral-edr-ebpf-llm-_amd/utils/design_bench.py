@@ -1,12 +1,13 @@
-"""Throughput of a hybrid design (Zokunex, Kalesun, Tugovik) beside the framework's other models at equal width and depth:
+"""Throughput of a hybrid design (Zokunex, Kalesun, Tugovik, Vogerax) beside the framework's other models at equal width and depth:
 whole-model prefill and decode steps, and each of the design's kernels beside its closest existing kernel with the
 fraction of its roofline it reaches.
 
-``python bench.py --design-compare [--design zokunex|kalesun|tugovik] [--design-sizes 1k,2k,4k]`` prints one JSON line
+``python bench.py --design-compare [--design zokunex|kalesun|tugovik|vogerax] [--design-sizes 1k,2k,4k]`` prints one JSON line
 (the default benchmark and its output line are untouched).  Zokunex stands beside Llama; Kalesun beside Zokunex (the
 closest family: recurrent layers, attention and mixtures of experts on a float32 stream) and Llama; Tugovik beside
 Kalesun (masked grouped-query attention over paged keys and values, linear-state scans behind a short convolution,
-gated experts, RMS norms on the stream) and Llama.  Weights are random; every number is measured on the GPU this
+gated experts, RMS norms on the stream) and Llama; Vogerax beside Kalesun too (windowed and causal sink attention on
+the same kernels, a linear-state scan, RMS norms joined to a float32 stream) and Llama.  Weights are random; every number is measured on the GPU this
 process runs on.
 
 Rooflines: HBM 8 TB/s for kernels bound by the bytes they must move, 2.5 PFLOP/s dense bf16 for the matrix-shaped
@@ -16,6 +17,7 @@ decode, like the Llama kernels they stand beside).
 from __future__ import annotations
 
 import json
+import math
 import sys
 import time
 
@@ -96,6 +98,34 @@ def tugovik_config(size: dict) -> dict:
     layers = [dict(mix_m, mlp=moe), dict(mix_a, mlp=moe), dict(mix_r, mlp=moe), dict(mix_a, mlp=moe)][:LAYERS]
     return dict(architecture="Tugovik", vocab=VOCAB, width=size["width"], norm=dict(eps=1e-6), layers=layers,
                 token_side=dict(dim=size["side"]))
+
+# Vogerax: width -> (pooled attention heads, kv heads, dim, window, pool | sink attention heads, kv heads, dim, vdim |
+#                    retention heads, dim, vdim | dense ff | experts, top, expert ff, shared ff | norm groups)
+VOGERAX_SIZES = {
+    "1k": dict(width=1024, a=(8, 2, 128, 512, 64), l=(8, 2, 128, 128), r=(8, 128, 128), ff=4096, moe=(8, 2, 512, 1024), groups=4),
+    "2k": dict(width=2048, a=(16, 4, 128, 1024, 64), l=(16, 4, 128, 128), r=(16, 128, 128), ff=8192, moe=(16, 4, 1024, 2048), groups=4),
+    "4k": dict(width=4096, a=(32, 8, 128, 1024, 64), l=(32, 8, 128, 128), r=(32, 128, 128), ff=14336, moe=(32, 4, 1536, 4096), groups=4),
+}
+
+
+def vogerax_config(size: dict) -> dict:
+    ah, ag, ad, win, pool = size["a"]
+    lh, lg, ld, lv = size["l"]
+    rh, rd, rv = size["r"]
+    ne, top, eff, sff = size["moe"]
+    mix_a = dict(type="attention", mixer=dict(heads=ah, kv_heads=ag, dim=ad, vdim=ad, scale=ad ** -0.5,
+                                              mask=dict(size=win, pool=pool),
+                                              rot=dict(base=5e5, dims=ad // 2, scaling=dict(factor=4.0))))
+    left = dict(heads=lh, kv_heads=lg, dim=ld, vdim=lv, scale=ld ** -0.5,
+                rot=dict(base=1e5, dims=ld // 2, scaling=dict(factor=8.0, original=4096, fast=16.0, slow=2.0)))
+    right = dict(heads=rh, dim=rd, vdim=rv, rot=dict(base=1e4, dims=rd),
+                 decay=[math.exp(-1.0 / (16.0 * 128.0 ** (h / max(1, rh - 1)))) for h in range(rh)])
+    mix_p = dict(type="parallel", mixer=dict(left=left, right=right))
+    dense = dict(kind="dense", ff=size["ff"])
+    moe = dict(kind="moe", expert=dict(ff=eff), shared=dict(ff=sff), router=dict(experts=ne, top=top))
+    layers = [dict(mix_a, mlp=dense), dict(mix_p, mlp=moe), dict(mix_a, mlp=moe), dict(mix_p, mlp=dense)][:LAYERS]
+    return dict(architecture="Vogerax", vocab=VOCAB, width=size["width"], norm=dict(eps=1e-6, groups=size["groups"]),
+                embedding=dict(scale=8.0), layers=layers)
 
 
 def _say(msg: str) -> None:
@@ -595,6 +625,205 @@ def run_tugovik(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ct
                 dtype="bf16", data="synthetic", sizes=res)
 
 
+def _kernels_vogerax(size: dict, ksize: dict, dev, T: int, ctx: int, rows: int) -> dict:
+    """Vogerax's kernels and their closest existing kernels at this size: seconds, and the fraction of the roofline
+    reached.  ``ksize``: the Kalesun sizes of the same width (for the kernels it stands beside)."""
+    from chronos import ops
+    from chronos.models.hybrid import rope_cos_sin
+    from chronos.ops import hybrid as hops
+
+    out = {}
+    bf = torch.bfloat16
+    d, ng = size["width"], size["groups"]
+    g = torch.Generator(device=dev).manual_seed(1)
+    rnd = lambda *s, dt=bf, sc=1.0: (torch.randn(*s, device=dev, generator=g) * sc).to(dt)  # noqa: E731
+    i32 = dict(dtype=torch.int32, device=dev)
+
+    def rec(name, secs, nbytes=0.0, flops=0.0):
+        roof = max(nbytes / HBM_BPS, flops / BF16_FLOPS)
+        _say(f"  {name}: {secs * 1e6:.1f} us, roofline {roof * 1e6:.2f} us")
+        out[name] = dict(us=round(secs * 1e6, 1), roofline_us=round(roof * 1e6, 2), of_roofline=round(roof / secs, 4))
+
+    bs = 16
+    seqs = max(1, T // ctx)
+    per = ctx // bs + 1
+    nb = max(seqs, rows) * per + 1
+    bt = torch.arange(1, 1 + seqs * per, **i32).view(seqs, per)
+    qs = torch.arange(0, (seqs + 1) * ctx, ctx, **i32)
+    pos = torch.arange(ctx, **i32).repeat(seqs)
+    tseq = torch.arange(seqs, **i32).repeat_interleave(ctx)
+    btd = torch.arange(1, 1 + rows * per, **i32).view(rows, per)
+    qsd = torch.arange(rows + 1, **i32)
+    posd = torch.full((rows,), ctx, **i32)
+    NS = max(seqs, rows) + 1
+    p0, sl, sld = torch.zeros(seqs, **i32), torch.arange(seqs, **i32), torch.arange(rows, **i32)
+    # ---- the stream's joins: norm of the addend, add, norm for the next sublayer, in one kernel
+    y, y2, x32 = rnd(T, d), rnd(T, d), rnd(T, d, dt=torch.float32)
+    w1, w2, w3, w4 = (rnd(d, dt=torch.float32) for _ in range(4))
+    rec("sandwich_join", _time(lambda: hops.sandwich_join(y, x32, w1, w2, ng, 1e-5, bf)), T * d * (2 + 4 + 4 + 2))
+    rec("sandwich_join.two_addends", _time(lambda: hops.sandwich_join(y, x32, w1, w2, ng, 1e-5, bf, y2)), T * d * (2 + 2 + 4 + 4 + 2))
+    rec("sandwich_join.pair", _time(lambda: hops.sandwich_join(y, x32, w1, w2, ng, 1e-5, bf, y2, (w3, w4))), T * d * (2 + 2 + 4 + 4 + 2))
+    yd, y2d, xd = rnd(rows, d), rnd(rows, d), rnd(rows, d, dt=torch.float32)
+    rec("sandwich_join.pair.decode", _time(lambda: hops.sandwich_join(yd, xd, w1, w2, ng, 1e-5, bf, y2d, (w3, w4))), rows * d * 14.0)
+    rec("kalesun.scale_add_rms_norm", _time(lambda: hops.scale_add_rms_norm(y, x32, w1, 1.0, 1e-6, bf)), T * d * (2 + 4 + 4 + 2))
+    rec("tugovik.add_rms_norm.normed_addend", _time(lambda: hops.add_rms_norm(y, x32, w1, 1e-6, bf, w_y=w2)), T * d * (2 + 4 + 4 + 2))
+    xb, wb = rnd(T, d), rnd(d)
+    rec("llama.add_rmsnorm", _time(lambda: ops.add_rmsnorm(y, xb, wb, 1e-5)), T * d * (2 + 2 + 2 + 2))
+    # ---- pooled-window attention beside Kalesun's window of the same span (with sink and gate) and Llama's
+    H, G, D, win, pool = size["a"]
+    ep = (bs + pool - 1) // pool
+    kc, vc = rnd(nb, bs, G, D, sc=0.3), rnd(nb, bs, G, D, sc=0.3)
+    kp, vp = rnd(nb, ep, G, D, sc=0.3), rnd(nb, ep, G, D, sc=0.3)
+    C = (H + G) * D
+    qk = rnd(seqs * ctx, C, sc=0.3)
+    tab = rope_cos_sin(5e5, D // 2, ctx + 2, dev, ("linear", 4.0))
+    vis = sum(min(i + 1, win) + max(0, i - win + 1) // pool for i in range(ctx))
+    rec("pooled_attention.prefill", _time(lambda: hops.window_attention(qk, kc, vc, bt, qs, pos, None, None, D ** -0.5, win, 0, H, bf, ctx, 0, pool, kp, vp), iters=3, warm=1),
+        flops=4.0 * seqs * vis * H * D)
+    rec("window_prep.values_are_keys.prefill", _time(lambda: hops.window_prep(qk, H, G, D, D, None, None, pos, tseq, bt, None, None, 1e-5, tab, D // 2, kc, vc, False, H * D)),
+        nbytes=seqs * ctx * (2 * (H + G) * D + 2 * G * D) * 2.0)
+    rec("pool_blocks.prefill", _time(lambda: hops.pool_blocks(kc, vc, kp, vp, bt, qs, p0, pool, ctx)),
+        nbytes=seqs * ctx * 2 * G * D * 2.0 * (1 + 1.0 / pool))
+    qkd = rnd(rows, C, sc=0.3)
+    rec("pooled_attention.decode", _time(lambda: hops.window_attention(qkd, kc, vc, btd, qsd, posd, None, None, D ** -0.5, win, 0, H, bf, 1, 0, pool, kp, vp)),
+        nbytes=rows * (min(ctx + 1, win) + max(0, ctx - win + 1) // pool) * G * 2 * D * 2.0)
+    rec("pool_blocks.decode", _time(lambda: hops.pool_blocks(kc, vc, kp, vp, btd, qsd, posd, pool, 1)), nbytes=1.0)
+    kH, kG, kD, kDv, kwin, keep = ksize["a"]
+    kkc, kvc = rnd(nb, bs, kG, kD, sc=0.3), rnd(nb, bs, kG, kDv, sc=0.3)
+    kqkv = rnd(seqs * ctx, (kH + kG) * kD + kG * kDv, sc=0.3)
+    kgate, ksink = rnd(seqs * ctx, kH, dt=torch.float32), rnd(kH, dt=torch.float32)
+    kvis = sum(min(i + 1, kwin) + max(0, min(keep, i + 1 - kwin)) for i in range(ctx))
+    rec("kalesun.window_attention.prefill", _time(lambda: hops.window_attention(kqkv, kkc, kvc, bt, qs, pos, ksink, kgate, kD ** -0.5, kwin, keep, kH, bf, ctx), iters=3, warm=1),
+        flops=2.0 * seqs * kvis * kH * (kD + kDv))
+    kqkvd, kgated = rnd(rows, (kH + kG) * kD + kG * kDv, sc=0.3), rnd(rows, kH, dt=torch.float32)
+    rec("kalesun.window_attention.decode", _time(lambda: hops.window_attention(kqkvd, kkc, kvc, btd, qsd, posd, ksink, kgated, kD ** -0.5, kwin, keep, kH, bf, 1)),
+        nbytes=rows * (min(ctx + 1, kwin) + keep) * kG * (kD + kDv) * 2.0)
+    # ---- causal sink attention with rotated values and a gate per column, beside Llama's causal attention
+    lH, lG, lD, lDv = size["l"]
+    lkc, lvc = rnd(nb, bs, lG, lD, sc=0.3), rnd(nb, bs, lG, lDv, sc=0.3)
+    Cl = (lH + lG) * lD + lG * lDv + lH * lDv
+    lq = rnd(seqs * ctx, Cl, sc=0.3)
+    lsink = rnd(lH, dt=torch.float32)
+    vtab = rope_cos_sin(1e5, lDv, ctx + 2, dev)
+    ltab = rope_cos_sin(1e5, lD // 2, ctx + 2, dev, ("ramp", 8.0, 4096.0, 16.0, 2.0))
+    qn, kn = rnd(lD, dt=torch.float32), rnd(lD, dt=torch.float32)
+    full_pairs = seqs * ctx * (ctx + 1) / 2
+    lg_off = (lH + lG) * lD + lG * lDv   # outputs turned back and gated per column in the attention's epilogue
+    rec("sink_attention.prefill", _time(lambda: hops.window_attention(lq, lkc, lvc, bt, qs, pos, lsink, None, lD ** -0.5, 0, 0, lH, bf, ctx, 0, 0, None, None, vtab, lg_off), iters=3, warm=1),
+        flops=2.0 * full_pairs * lH * (lD + lDv))
+    rec("window_prep.rotated_values.prefill", _time(lambda: hops.window_prep(lq, lH, lG, lD, lDv, None, None, pos, tseq, bt, qn, kn, 1e-5, ltab, lD // 2, lkc, lvc, False, -1, vtab)),
+        nbytes=seqs * ctx * (2 * (lH + lG) * lD + 2 * lG * lDv) * 2.0)
+    lo = rnd(seqs * ctx, lH * lDv)
+    rec("unrotate_gate.prefill", _time(lambda: hops.unrotate_gate(lo, pos, vtab, lq, (lH + lG) * lD + lG * lDv, lH, lDv, bf)),
+        nbytes=seqs * ctx * lH * lDv * 6.0)
+    lqd = rnd(rows, Cl, sc=0.3)
+    rec("sink_attention.decode", _time(lambda: hops.window_attention(lqd, lkc, lvc, btd, qsd, posd, lsink, None, lD ** -0.5, 0, 0, lH, bf, 1, 0, 0, None, None, vtab, lg_off)),
+        nbytes=rows * (ctx + 1) * lG * (lD + lDv) * 2.0)
+    hq = d // 128
+    hkv = max(1, hq // 4)
+    akc, avc = rnd(nb, hkv, bs, 128, sc=0.3), rnd(nb, hkv, 128, bs, sc=0.3)
+    q = rnd(seqs * ctx, hq, 128, sc=0.3)
+    ctxl = torch.full((seqs,), ctx, **i32)
+    tiles = torch.tensor(ops.attention_tiles([ctx] * seqs, hq, hkv, 8), **i32).view(-1, 2)
+    rec("llama.attention.prefill", _time(lambda: ops.paged_attention(q, akc, avc, bt, qs, ctxl, tiles, tiles.shape[0], 8, 1), iters=3, warm=1),
+        flops=4.0 * full_pairs * hq * 128)
+    qd = rnd(rows, hq, 128, sc=0.3)
+    ctxd = torch.full((rows,), ctx + 1, **i32)
+    ns = ops.pick_nsplit(rows * hkv, ctx + 1)
+    rec("llama.attention.decode", _time(lambda: ops.paged_attention(qd, akc, avc, btd, qsd, ctxd, None, rows, 1, ns)),
+        nbytes=rows * (ctx + 1) * hkv * 128 * 2 * 2.0)
+    # ---- retention: the linear-state scan with fixed decays beside Kalesun's gated linear attention on the same kernel
+    rh, rd, rv = size["r"]
+    Cr = 2 * rh * rd + 2 * rh * rv
+    S = torch.zeros(NS, rh, rd, rv, device=dev)
+    dec = torch.tensor([math.exp(-1.0 / (16.0 * 128.0 ** (h / max(1, rh - 1)))) for h in range(rh)], device=dev)
+    rtab = rope_cos_sin(1e4, rd, ctx + 2, dev)
+    ones = torch.ones(rh * rv, device=dev)
+    proj, projd = rnd(seqs * ctx, Cr, sc=0.5), rnd(rows, Cr, sc=0.5)
+    rec("rotate_qk.prefill", _time(lambda: hops.rotate_qk(proj, 0, rh * rd, rh, rh, rd, rd, rtab, pos, 1.0, 1.0)), nbytes=seqs * ctx * 2 * rh * rd * 4.0)
+    rec("retention_scan.prefill", _time(lambda: hops.linear_scan(proj, 0, rh * rd, 2 * rh * rd, None, None, 1.0, dec, None, qs, p0, sl, S, rh, rh, rd, rv), iters=3, warm=1),
+        nbytes=seqs * ctx * Cr * 2.0, flops=seqs * ctx * rh * rd * rv * 4.0)
+    rec("retention_scan.decode", _time(lambda: hops.linear_scan(projd, 0, rh * rd, 2 * rh * rd, None, None, 1.0, dec, None, qsd, posd, sld, S, rh, rh, rd, rv)),
+        nbytes=rows * rh * rd * rv * 4 * 2.0)
+    o32 = rnd(seqs * ctx, rh, rv, dt=torch.float32)
+    rec("head_norm_gate.prefill", _time(lambda: hops.head_norm_gate(o32, proj, 2 * rh * rd + rh * rv, ones, 1e-5, True, bf)), nbytes=seqs * ctx * rh * rv * 8.0)
+    gh, gd, gv = ksize["g"]
+    gS = torch.zeros(NS, gh, gd, gv, device=dev)
+    gproj, gprojd = rnd(seqs * ctx, 2 * gh * gd + gh * gv, sc=0.5), rnd(rows, 2 * gh * gd + gh * gv, sc=0.5)
+    gdec, gdecd = torch.rand(seqs * ctx, gh, gd, device=dev), torch.rand(rows, gh, gd, device=dev)
+    rec("kalesun.linear_scan.gla.prefill", _time(lambda: hops.linear_scan(gproj, 0, gh * gd, 2 * gh * gd, None, None, gd ** -0.5, gdec, None, qs, p0, sl, gS, gh, gh, gd, gv), iters=3, warm=1),
+        nbytes=seqs * ctx * (2 * gh * gd + gh * gv) * 2.0, flops=seqs * ctx * gh * gd * gv * 4.0)
+    rec("kalesun.linear_scan.gla.decode", _time(lambda: hops.linear_scan(gprojd, 0, gh * gd, 2 * gh * gd, None, None, gd ** -0.5, gdecd, None, qsd, posd, sld, gS, gh, gh, gd, gv)),
+        nbytes=rows * gh * gd * gv * 4 * 2.0)
+    # ---- feed-forwards: squared-ReLU experts behind a softmax router beside Kalesun's gated experts and Llama's MLP
+    ne, top, eff, sff = size["moe"]
+    wr, corr = rnd(ne, d, sc=0.05), torch.zeros(ne, device=dev)
+    wu, wd = rnd(ne, eff, d, sc=d ** -0.5), rnd(ne, d, eff, sc=eff ** -0.5)
+    kne, ktop, keff = ksize["moe"]
+    kwr, kbr = rnd(kne, d, sc=0.05), rnd(kne, dt=torch.float32, sc=0.01)
+    kwgu = rnd(kne, 2 * keff, d, sc=d ** -0.5)[:, hops.moe_glu_row_order(keff).to(dev)].contiguous()
+    kwd = rnd(kne, d, keff, sc=keff ** -0.5)
+    for name, tk in (("prefill", T), ("decode", rows)):
+        h = rnd(tk, d)
+        idx, wt = hops.moe_route(h, wr, corr, top)
+        rec(f"moe_route.{name}", _time(lambda: hops.moe_route(h, wr, corr, top)), nbytes=tk * d * 2.0 + ne * d * 2.0)
+        rec(f"moe_ffn.relu2.{name}", _time(lambda: hops.moe_ffn(h, idx, wt, wu, wd, hops.ACT_RELU2, bf), iters=3, warm=1),
+            nbytes=min(ne, tk * top) * 2 * eff * d * 2.0 + tk * d * 4.0, flops=tk * top * 4.0 * eff * d)
+        kidx, kwt = hops.moe_route_topk(h, kwr, kbr, ktop)
+        rec(f"kalesun.moe_route_topk.{name}", _time(lambda: hops.moe_route_topk(h, kwr, kbr, ktop)), nbytes=tk * d * 2.0 + kne * d * 2.0)
+        rec(f"kalesun.moe_glu_ffn.{name}", _time(lambda: hops.moe_glu_ffn(h, kidx, kwt, kwgu, kwd, 7.0, 1.702, 1.0, bf, True), iters=3, warm=1),
+            nbytes=min(kne, tk * ktop) * 3 * keff * d * 2.0 + tk * d * 4.0, flops=tk * ktop * 6.0 * keff * d)
+        lf = int(3.5 * d)
+        wgl, wdn = rnd(2 * lf, d, sc=d ** -0.5), rnd(d, lf, sc=lf ** -0.5)
+        rec(f"llama.mlp.{name}", _time(lambda: ops.linear(ops.gate_up_silu(h, wgl), wdn), iters=3, warm=1),
+            nbytes=3 * lf * d * 2.0 + tk * d * 4.0, flops=tk * 6.0 * lf * d)
+    return out
+
+
+def run_vogerax(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int = 2048, device: str = "cuda") -> dict:
+    from chronos import ops
+    from chronos.models import kalesun, llama, vogerax
+    from chronos.models.hybrid import HybridDecoder
+
+    dev = torch.device(device if ":" in device else device + ":0")
+    torch.cuda.set_device(dev)
+    ops.load()
+    ops.device_init()
+    res = {}
+    P = ctx + plen + 16
+    for name in sizes:
+        size, ksize = VOGERAX_SIZES[name], KALESUN_SIZES[name]
+        t0 = time.time()
+        cfg = vogerax.config_from_dict(vogerax_config(size), name=f"vogerax-{name}", max_position=P)
+        vm = HybridDecoder(cfg, vogerax.pack_weights(cfg, vogerax.random_tensors(cfg, 0), dev, torch.bfloat16), dev, P,
+                           torch.bfloat16)
+        entry = dict(vogerax=dict(params=cfg.param_count(), **_model_steps(vm, dev, seqs, plen, rows, ctx)))
+        _say(f"size {name}: vogerax {entry['vogerax']}")
+        del vm
+        kcfg = kalesun.config_from_dict(kalesun_config(ksize), name=f"kalesun-{name}", max_position=P)
+        km = HybridDecoder(kcfg, kalesun.pack_weights(kcfg, kalesun.random_tensors(kcfg, 0), dev, torch.bfloat16), dev, P,
+                           torch.bfloat16)
+        entry["kalesun"] = dict(params=kcfg.param_count(), **_model_steps(km, dev, seqs, plen, rows, ctx))
+        _say(f"  kalesun {entry['kalesun']}")
+        del km
+        d = size["width"]
+        lc = llama.LlamaConfig(name=f"llama-{name}", vocab_size=VOCAB, hidden_size=d, intermediate_size=int(3.5 * d),
+                               num_layers=LAYERS, num_heads=d // 128, num_kv_heads=max(1, d // 512), max_position=P)
+        lm = llama.LlamaModel(lc, llama.random_weights(lc, None, dev, 0), None, dev, P)
+        entry["llama"] = dict(params=lc.param_count(), **_model_steps(lm, dev, seqs, plen, rows, ctx))
+        _say(f"  llama {entry['llama']}")
+        del lm
+        torch.cuda.empty_cache()
+        entry["kernels"] = _kernels_vogerax(size, ksize, dev, seqs * plen, ctx, rows)
+        entry["seconds"] = round(time.time() - t0, 1)
+        res[name] = entry
+        torch.cuda.empty_cache()
+    return dict(metric="design_compare", design="vogerax", beside="kalesun and llama (equal width and depth)",
+                layers=LAYERS, workload=dict(prefill=f"{seqs} x {plen} tokens in one step",
+                                             decode=f"{rows} rows at context {ctx}"),
+                dtype="bf16", data="synthetic", sizes=res)
+
+
 def run_kalesun(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int = 2048, device: str = "cuda") -> dict:
     from chronos import ops
     from chronos.models import kalesun, llama, zokunex
@@ -677,7 +906,7 @@ def run(sizes: list, seqs: int = 4, plen: int = 2048, rows: int = 64, ctx: int =
 
 def main(a) -> int:
     sizes = [s for s in a.design_sizes.split(",") if s]
-    fn = {"kalesun": run_kalesun, "tugovik": run_tugovik}.get(getattr(a, "design", "zokunex"), run)
+    fn = {"kalesun": run_kalesun, "tugovik": run_tugovik, "vogerax": run_vogerax}.get(getattr(a, "design", "zokunex"), run)
     out = fn(sizes, device=a.device)
     print(json.dumps(out), flush=True)
     return 0
